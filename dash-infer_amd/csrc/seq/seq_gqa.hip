@@ -6,6 +6,11 @@
 //   gqa_attn_mc_kernel + merge   bf16 caches on the matrix cores, the key walk split for few rows (decoding)
 // Options of the softmax: a sink logit per head or the constant 0 (one more term in the denominator, no value), a tanh cap on
 // the scores, a multiplier per (row, head) on the output (the output gate).
+// Options of the key walk: a sliding window with kept first keys (row p reads key j <= p if p - j < window or j < keep_first;
+// the keys between are skipped by whole chunks / tiles), and several softmax maps per head (`maps`: head h has maps query
+// vectors and its key head maps key vectors, laid out one after the other; map m of a head scores against map m of its key
+// head, all maps read the same values; the output holds the maps of a head side by side).
+//   maps_diff_norm    two maps per head -> one: (first - lam * second) / its root mean square * a constant
 #include "seq_common.h"
 
 namespace dihip {
@@ -14,7 +19,7 @@ namespace {
 // ------------------------------------------------------------------------------------------------ prep + append
 struct PrepArgs {
   float* qkv; long ld; int q_off, k_off, v_off;
-  int H, G, D, DV;
+  int H, G, D, DV, GV;   // H / G: query / key vectors per token (heads x maps), GV: value heads
   const void* qnorm; const void* knorm; int wdt; float eps;
   const float* freq; int rot_dims, layout; float mag;
   float lam; const float* vfirst_in; float* vfirst_out; long ldvf;
@@ -84,7 +89,7 @@ __global__ __launch_bounds__(256) void qkv_prep_append_kernel(PrepArgs a) {
     }
   }
   void* vdst = a.vspans[sp];
-  const int nv = a.G * a.DV;
+  const int nv = a.GV * a.DV;
   for (int e = blockIdx.y * 256 + threadIdx.x; e < nv; e += 256 * gridDim.y) {
     float v = row[a.v_off + e];
     if (a.vfirst_in) v = (1.f - a.lam) * v + a.lam * a.vfirst_in[(size_t)t * a.ldvf + e];
@@ -104,83 +109,115 @@ struct GqaArgs {
   const int32_t* tok_slot; const int32_t* tok_pos; const int32_t* ent_slot; const int32_t* ent_row0; const int32_t* ent_count;
   int H, G, D, DV; float scale;
   float* ws; int rows_total;
+  int maps, window, keep_first;           // window <= 0: every key up to the row's own
 };
 
 __device__ __forceinline__ float cap_score(float s, float cap) { return cap > 0.f ? cap * tanhf(s / cap) : s; }
 
-// One workgroup per row, its 4 waves take the heads in turn; a wave walks the keys 64 at a time: lane j scores key j (d
-// ascending), the chunk joins the running softmax, then the lanes turn to the value elements and add the weighted rows.
+// One workgroup per row, its 4 waves take the (head, map) pairs in turn; a wave walks the keys it may read 64 at a time (first the
+// kept first keys that lie before the window, then the window): lane j scores key j (d ascending), the chunk joins the running
+// softmax, then the lanes turn to the value elements and add the weighted rows.
 template <int CT, int RV>
 __global__ __launch_bounds__(256) void gqa_attn_kernel(GqaArgs a) {
   __shared__ float qs[4][256];
   __shared__ float ps[4][64];
   const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int pos = a.tok_pos[t], H = a.H, G = a.G, D = a.D, DV = a.DV, hpg = H / G;
+  const int pos = a.tok_pos[t], H = a.H, G = a.G, D = a.D, DV = a.DV, hpg = H / G, M = a.maps, HQ = H * M, GK = G * M;
+  const int w_lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;   // the window is [w_lo, pos]
+  const int first_hi = min(a.keep_first, w_lo);                     // the kept first keys before it: [0, first_hi)
   void* const* ktab = a.kspans + (size_t)a.tok_slot[t] * a.span_stride;
   void* const* vtab = a.vspans + (size_t)a.tok_slot[t] * a.span_stride;
   constexpr size_t ES = CT == DIHIP_F32 ? 4 : 2;
-  for (int h0 = 0; h0 < H; h0 += 4) {
-    const int h = h0 + wave;
-    const bool live = h < H;
-    const int g = (live ? h : 0) / hpg;
+  for (int h0 = 0; h0 < HQ; h0 += 4) {
+    const int hq = h0 + wave;
+    const bool live = hq < HQ;
+    const int h = (live ? hq : 0) / M, mp = (live ? hq : 0) - h * M;
+    const int g = h / hpg, gk = g * M + mp;
     __syncthreads();
     if (live)
-      for (int d = lane; d < D; d += 64) qs[wave][d] = a.q[(size_t)t * a.ldq + (size_t)h * D + d];
+      for (int d = lane; d < D; d += 64) qs[wave][d] = a.q[(size_t)t * a.ldq + (size_t)hq * D + d];
     __syncthreads();
     float mx = -INFINITY, den = 0.f;
-    if (a.sink_mode == 1) { mx = ld_any(a.sink, live ? h : 0, a.wdt); den = 1.f; }
+    if (a.sink_mode == 1) { mx = ld_any(a.sink, h, a.wdt); den = 1.f; }
     else if (a.sink_mode == 2) { mx = 0.f; den = 1.f; }
     float acc[RV];
 #pragma unroll
     for (int v = 0; v < RV; ++v) acc[v] = 0.f;
-    for (int j0 = 0; j0 <= pos; j0 += 64) {
-      const int j = j0 + lane;
-      const bool valid = live && j <= pos;
-      float s = -INFINITY;
-      if (valid) {
-        const char* kr = (const char*)ktab[j / a.span_len] + ((size_t)(j % a.span_len) * G + g) * D * ES;
-        float d = 0.f;
-        for (int r = 0; r < D; ++r) d = __builtin_fmaf(qs[wave][r], load_ft<CT>(kr, r), d);
-        s = cap_score(d * a.scale, a.softcap);
-      }
-      const float mnew = fmaxf(mx, wave_max(s));
-      const float corr = mx == -INFINITY ? 0.f : expf(mx - mnew);
-      const float p = valid ? expf(s - mnew) : 0.f;
-      den = den * corr + wave_sum(p);
+    for (int part = 0; part < 2; ++part) {                       // the same trip counts in every wave of the block
+      const int r_lo = part ? w_lo : 0, r_hi = part ? pos + 1 : first_hi;
+      for (int j0 = r_lo; j0 < r_hi; j0 += 64) {
+        const int j = j0 + lane;
+        const bool valid = live && j < r_hi;
+        float s = -INFINITY;
+        if (valid) {
+          const char* kr = (const char*)ktab[j / a.span_len] + ((size_t)(j % a.span_len) * GK + gk) * D * ES;
+          float d = 0.f;
+          for (int r = 0; r < D; ++r) d = __builtin_fmaf(qs[wave][r], load_ft<CT>(kr, r), d);
+          s = cap_score(d * a.scale, a.softcap);
+        }
+        const float mnew = fmaxf(mx, wave_max(s));
+        const float corr = mx == -INFINITY ? 0.f : expf(mx - mnew);
+        const float p = valid ? expf(s - mnew) : 0.f;
+        den = den * corr + wave_sum(p);
 #pragma unroll
-      for (int v = 0; v < RV; ++v) acc[v] *= corr;
-      mx = mnew;
-      ps[wave][lane] = p;
-      __syncthreads();
-      if (live) {
-        const int cnt = min(64, pos - j0 + 1);
-        for (int jj = 0; jj < cnt; ++jj) {
-          const int jk = j0 + jj;
-          const char* vr = (const char*)vtab[jk / a.span_len] + ((size_t)(jk % a.span_len) * G + g) * DV * ES;
-          const float pj = ps[wave][jj];
+        for (int v = 0; v < RV; ++v) acc[v] *= corr;
+        mx = mnew;
+        ps[wave][lane] = p;
+        __syncthreads();
+        if (live) {
+          const int cnt = min(64, r_hi - j0);
+          for (int jj = 0; jj < cnt; ++jj) {
+            const int jk = j0 + jj;
+            const char* vr = (const char*)vtab[jk / a.span_len] + ((size_t)(jk % a.span_len) * G + g) * DV * ES;
+            const float pj = ps[wave][jj];
 #pragma unroll
-          for (int v = 0; v < RV; ++v) {
-            const int r = v * 64 + lane;
-            if (r < DV) acc[v] = __builtin_fmaf(pj, load_ft<CT>(vr, r), acc[v]);
+            for (int v = 0; v < RV; ++v) {
+              const int r = v * 64 + lane;
+              if (r < DV) acc[v] = __builtin_fmaf(pj, load_ft<CT>(vr, r), acc[v]);
+            }
           }
         }
+        __syncthreads();
       }
-      __syncthreads();
     }
     if (live) {
       const float gt = a.gate ? a.gate[(size_t)t * a.ldg + h] : 1.f;
 #pragma unroll
       for (int v = 0; v < RV; ++v) {
         const int r = v * 64 + lane;
-        if (r < DV) a.out[(size_t)t * a.ldo + (size_t)h * DV + r] = acc[v] / den * gt;
+        if (r < DV) a.out[(size_t)t * a.ldo + (size_t)hq * DV + r] = acc[v] / den * gt;
       }
     }
   }
 }
 
+// Two maps per head -> one: d = first - lam * second, out = d / sqrt(mean(d^2) + eps) * out_scale.  A wave per (row, head).
+__global__ __launch_bounds__(256) void maps_diff_norm_kernel(void* __restrict__ y, int ydt, long ldy, const float* __restrict__ x, long ldx,
+                                                             float lam, float out_scale, float eps, int TH, int H, int DV) {
+  const int pair = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (pair >= TH) return;
+  const int t = pair / H, h = pair - t * H;
+  const float* a1 = x + (size_t)t * ldx + (size_t)h * 2 * DV;
+  const float* a2 = a1 + DV;
+  float v[8], ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int d = lane + 64 * i;
+    v[i] = d < DV ? a1[d] - lam * a2[d] : 0.f;
+    ss = __builtin_fmaf(v[i], v[i], ss);
+  }
+  const float inv = out_scale / sqrtf(wave_sum(ss) / (float)DV + eps);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int d = lane + 64 * i;
+    if (d < DV) st_any(y, (size_t)t * ldy + (size_t)h * DV + d, ydt, v[i] * inv);
+  }
+}
+
 // ------------------------------------------------------------------------------------------------ matrix-core kernel
-// A workgroup owns 64 consecutive (row, query head) pairs of ONE portion and ONE key/value head -- 16 per wave -- and walks
-// the 32-key tiles those pairs can see.  Per tile: S^T = K . Q^T (the tile's key rows as they lie in LDS against the wave's
+// A workgroup owns 64 consecutive (row, query head) pairs of ONE portion, ONE key/value head and ONE map -- 16 per wave -- and
+// walks the 32-key tiles those pairs can see (with a window: the tiles of the kept first keys, then those from the window of its
+// first row on).  Per tile: S^T = K . Q^T (the tile's key rows as they lie in LDS against the wave's
 // query fragments, held in registers for the whole walk), cap + mask + running softmax on the accumulator lanes, then
 // O^T += V^T . P^T with P straight from those lanes and V^T read from the value tile through the transposing LDS read.  The
 // next tile's rows are in flight meanwhile.  Head sizes that are no multiple of the tile's granule are padded with zero
@@ -195,7 +232,8 @@ __global__ __launch_bounds__(256) void gqa_attn_mc_kernel(GqaArgs a) {
   constexpr int KS = DMAX / 32, DT = VMAX / 16, UNK = DMAX / 64, UNV = VMAX / 64;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int G = a.G, H = a.H, D = a.D, DV = a.DV, hpg = H / G;
-  const int e = blockIdx.y / G, g = blockIdx.y - e * G, split = blockIdx.z, nsplit = gridDim.z;
+  const int M = a.maps, GK = G * M;
+  const int e = blockIdx.y / GK, gk = blockIdx.y - e * GK, g = gk / M, mp = gk - g * M, split = blockIdx.z, nsplit = gridDim.z;
   const int cnt = a.ent_count[e], row0 = a.ent_row0[e];
   const int nrows = cnt * hpg, r0 = blockIdx.x * 64;
   if (r0 >= nrows) return;
@@ -208,15 +246,19 @@ __global__ __launch_bounds__(256) void gqa_attn_mc_kernel(GqaArgs a) {
   const int myrow = r0 + wave * 16 + ni;
   const bool row_ok = myrow < nrows;
   const int rr = row_ok ? myrow : nrows - 1;
-  const int tq = rr / hpg, h = g * hpg + (rr - tq * hpg), p = pos0 + tq;
-  const int p_hi = pos0 + min(r0 + 63, nrows - 1) / hpg;
+  const int tq = rr / hpg, h = g * hpg + (rr - tq * hpg), hq = h * M + mp, p = pos0 + tq;
+  const int p_lo = pos0 + r0 / hpg, p_hi = pos0 + min(r0 + 63, nrows - 1) / hpg;
   const int tile_hi = p_hi >> 5;
-  const int per = (tile_hi + nsplit) / nsplit;
-  const int my_lo = split * per, my_hi = min(tile_hi, my_lo + per - 1);
+  const int win_t0 = (a.window > 0 ? max(0, p_lo - a.window + 1) : 0) >> 5;          // the first tile of the window of the first row
+  const int n_first = min(win_t0, (min(a.keep_first, p_hi + 1) + 31) >> 5);           // tiles of kept first keys before it
+  const int n_tiles = n_first + tile_hi - win_t0 + 1;
+  const int per = (n_tiles + nsplit - 1) / nsplit;
+  const int my_lo = split * per, my_hi = min(n_tiles - 1, my_lo + per - 1);           // indices into the walk: tile_of(i)
+  auto tile_of = [&](int i) { return i < n_first ? i : win_t0 + (i - n_first); };
 
   u32x4_t qf[KS];
   {
-    const float* qrow = a.q + (size_t)(row0 + tq) * a.ldq + (size_t)h * D;
+    const float* qrow = a.q + (size_t)(row0 + tq) * a.ldq + (size_t)hq * D;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       qf[ks] = u32x4_t{0u, 0u, 0u, 0u};
@@ -247,13 +289,13 @@ __global__ __launch_bounds__(256) void gqa_attn_mc_kernel(GqaArgs a) {
   }
   __shared__ const char* ktabs[128];
   __shared__ const char* vtabs[128];
-  void* const* gk = a.kspans + (size_t)a.ent_slot[e] * a.span_stride;
+  void* const* gkp = a.kspans + (size_t)a.ent_slot[e] * a.span_stride;
   void* const* gv = a.vspans + (size_t)a.ent_slot[e] * a.span_stride;
-  const int span_lo = (my_lo * 32) / a.span_len;
+  const int span_lo = my_lo <= my_hi ? (tile_of(my_lo) * 32) / a.span_len : 0;
   for (int i = tid; i < 128; i += 256) {
     const int sp = span_lo + i;
     const bool in = sp * a.span_len <= p_hi;
-    ktabs[i] = in ? (const char*)gk[sp] : nullptr;
+    ktabs[i] = in ? (const char*)gkp[sp] : nullptr;
     vtabs[i] = in ? (const char*)gv[sp] : nullptr;
   }
   __syncthreads();
@@ -262,7 +304,7 @@ __global__ __launch_bounds__(256) void gqa_attn_mc_kernel(GqaArgs a) {
 #pragma unroll
   for (int j = 0; j < UNK; ++j) {
     const int u = tid + 256 * j, kin = u / uprk, c8 = u - kin * uprk;
-    gok[j] = kin < 32 ? ((kin * G + g) * D + c8 * 8) * 2 : -1;
+    gok[j] = kin < 32 ? ((kin * GK + gk) * D + c8 * 8) * 2 : -1;
     lok[j] = kin * pitchk + c8 * 16;
   }
 #pragma unroll
@@ -275,7 +317,7 @@ __global__ __launch_bounds__(256) void gqa_attn_mc_kernel(GqaArgs a) {
   auto fetch = [&](int tile) {
     const int key0 = tile * 32, sp = key0 / a.span_len, in = key0 - sp * a.span_len;
     const bool near = sp - span_lo < 128;
-    const char* kbp = (near ? ktabs[sp - span_lo] : (const char*)gk[sp]) + (size_t)in * G * D * 2;
+    const char* kbp = (near ? ktabs[sp - span_lo] : (const char*)gkp[sp]) + (size_t)in * GK * D * 2;
     const char* vbp = (near ? vtabs[sp - span_lo] : (const char*)gv[sp]) + (size_t)in * G * DV * 2;
 #pragma unroll
     for (int j = 0; j < UNK; ++j) {
@@ -288,8 +330,9 @@ __global__ __launch_bounds__(256) void gqa_attn_mc_kernel(GqaArgs a) {
       if (gov[j] >= 0) prev[j] = gload<u32x4_t>(vbp + gov[j]);
     }
   };
-  if (my_lo <= my_hi) fetch(my_lo);
-  for (int tile = my_lo; tile <= my_hi; ++tile) {
+  if (my_lo <= my_hi) fetch(tile_of(my_lo));
+  for (int ti = my_lo; ti <= my_hi; ++ti) {
+    const int tile = tile_of(ti);
 #pragma unroll
     for (int j = 0; j < UNK; ++j)
       if (gok[j] >= 0) *reinterpret_cast<u32x4_t*>(ksm + lok[j]) = prek[j];
@@ -297,7 +340,7 @@ __global__ __launch_bounds__(256) void gqa_attn_mc_kernel(GqaArgs a) {
     for (int j = 0; j < UNV; ++j)
       if (gov[j] >= 0) *reinterpret_cast<u32x4_t*>(vsm + lov[j]) = prev[j];
     __syncthreads();
-    if (tile + 1 <= my_hi) fetch(tile + 1);
+    if (ti + 1 <= my_hi) fetch(tile_of(ti + 1));
     f32x4_t sacc[2] = {z4, z4};
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
@@ -317,7 +360,8 @@ __global__ __launch_bounds__(256) void gqa_attn_mc_kernel(GqaArgs a) {
         const int key = tile * 32 + nt * 16 + kb * 4 + r;
         float s = sacc[nt][r] * a.scale;
         if (a.softcap > 0.f) s = a.softcap * fast_tanh(s / a.softcap);
-        sv[nt][r] = key <= p ? s : -INFINITY;
+        const bool seen = key <= p && (a.window <= 0 || p - key < a.window || key < a.keep_first);
+        sv[nt][r] = seen ? s : -INFINITY;
         mx = fmaxf(mx, sv[nt][r]);
       }
     mx = rows_max(mx);
@@ -357,12 +401,12 @@ __global__ __launch_bounds__(256) void gqa_attn_mc_kernel(GqaArgs a) {
   if (!row_ok) return;
   if (nsplit == 1) {
     const float inv = (a.gate ? a.gate[(size_t)(row0 + tq) * a.ldg + h] : 1.f) / l;
-    float* o = a.out + (size_t)(row0 + tq) * a.ldo + (size_t)h * DV + kb * 4;
+    float* o = a.out + (size_t)(row0 + tq) * a.ldo + (size_t)hq * DV + kb * 4;
 #pragma unroll
     for (int t = 0; t < DT; ++t)
       if (t * 16 + kb * 4 < DV) *reinterpret_cast<f32x4_t*>(o + t * 16) = f32x4_t{oacc[t][0] * inv, oacc[t][1] * inv, oacc[t][2] * inv, oacc[t][3] * inv};
   } else {
-    float* o = a.ws + ((size_t)split * a.rows_total + (size_t)(row0 + tq) * H + h) * (Vp + 4);
+    float* o = a.ws + ((size_t)split * a.rows_total + (size_t)(row0 + tq) * H * M + hq) * (Vp + 4);
 #pragma unroll
     for (int t = 0; t < DT; ++t)
       if (t * 16 < Vp) *reinterpret_cast<f32x4_t*>(o + t * 16 + kb * 4) = oacc[t];
@@ -372,10 +416,10 @@ __global__ __launch_bounds__(256) void gqa_attn_mc_kernel(GqaArgs a) {
 
 // one workgroup per (row, head): the splits' (maximum, denominator, sums) records -> the row's output
 __global__ __launch_bounds__(256) void gqa_attn_merge_kernel(float* __restrict__ out, long ldo, const float* __restrict__ ws, int nsplit,
-                                                             int rows_total, int H, int DV, int Vp, const float* __restrict__ gate, long ldg) {
+                                                             int rows_total, int H, int maps, int DV, int Vp, const float* __restrict__ gate, long ldg) {
   __shared__ float wgt[1024];
   __shared__ float red[4];
-  const int gi = blockIdx.x, t = gi / H, h = gi - t * H;
+  const int gi = blockIdx.x, HQ = H * maps, t = gi / HQ, hq = gi - t * HQ, h = hq / maps;
   const size_t rec = (size_t)Vp + 4, stride = (size_t)rows_total * rec;
   const float* base = ws + (size_t)gi * rec;
   float mloc[4], lloc[4], mx = -INFINITY;
@@ -404,7 +448,7 @@ __global__ __launch_bounds__(256) void gqa_attn_merge_kernel(float* __restrict__
     float acc = 0.f;
 #pragma unroll 8
     for (int s = 0; s < nsplit; ++s) acc = __builtin_fmaf(wgt[s], base[s * stride + r], acc);
-    out[(size_t)t * ldo + (size_t)h * DV + r] = acc * inv;
+    out[(size_t)t * ldo + (size_t)hq * DV + r] = acc * inv;
   }
 }
 
@@ -415,7 +459,7 @@ using namespace dihip;
 
 extern "C" {
 
-int dihip_qkv_prep_append(void* stream, float* qkv, long ld, int q_off, int k_off, int v_off, int H, int G, int D, int DV,
+int dihip_qkv_prep_append(void* stream, float* qkv, long ld, int q_off, int k_off, int v_off, int H, int G, int D, int DV, int maps,
                           const void* qnorm, const void* knorm, int w_dtype, float eps, const float* freq, int rot_dims, int layout,
                           float mag, float lam, const float* vfirst_in, float* vfirst_out, long ldvf, void* const* kspans,
                           void* const* vspans, int span_stride, int span_len, int cache_dtype, const int32_t* tok_slot,
@@ -423,13 +467,17 @@ int dihip_qkv_prep_append(void* stream, float* qkv, long ld, int q_off, int k_of
   DIHIP_REQUIRE(T >= 0 && qkv && H > 0 && G > 0 && H % G == 0 && D > 0 && D <= 256 && DV > 0 && kspans && vspans && tok_slot && tok_pos &&
                     span_stride > 0 && span_len > 0 && seq_dtype_ok(cache_dtype) && seq_dtype_ok(w_dtype), DIHIP_PARAM_ERROR,
                 "qkv_prep_append: bad argument (heads of at most 256 elements)");
+  DIHIP_REQUIRE(maps >= 1 && maps <= 8, DIHIP_PARAM_ERROR, "qkv_prep_append: 1 to 8 maps per head");
+  const int GV = G;
+  H *= maps;     // from here on: query / key vectors per token
+  G *= maps;
   DIHIP_REQUIRE(q_off >= 0 && k_off >= 0 && v_off >= 0 && ld >= (long)q_off + (long)H * D && ld >= (long)k_off + (long)G * D &&
-                    ld >= (long)v_off + (long)G * DV, DIHIP_PARAM_ERROR, "qkv_prep_append: columns outside the rows");
+                    ld >= (long)v_off + (long)GV * DV, DIHIP_PARAM_ERROR, "qkv_prep_append: columns outside the rows");
   DIHIP_REQUIRE(rot_dims >= 0 && rot_dims <= D && rot_dims % 2 == 0 && (rot_dims == 0 || freq) && (layout == 0 || layout == 1),
                 DIHIP_PARAM_ERROR, "qkv_prep_append: bad rotation (an even number of dimensions up to the head size, layout 0 / 1)");
-  DIHIP_REQUIRE((!vfirst_in && !vfirst_out) || ldvf >= (long)G * DV, DIHIP_PARAM_ERROR, "qkv_prep_append: value rows shorter than the values");
+  DIHIP_REQUIRE((!vfirst_in && !vfirst_out) || ldvf >= (long)GV * DV, DIHIP_PARAM_ERROR, "qkv_prep_append: value rows shorter than the values");
   if (T == 0) return DIHIP_SUCCESS;
-  PrepArgs a{qkv, ld, q_off, k_off, v_off, H, G, D, DV, qnorm, knorm, w_dtype, eps, freq, rot_dims, layout, mag, lam, vfirst_in, vfirst_out,
+  PrepArgs a{qkv, ld, q_off, k_off, v_off, H, G, D, DV, GV, qnorm, knorm, w_dtype, eps, freq, rot_dims, layout, mag, lam, vfirst_in, vfirst_out,
              ldvf, kspans, vspans, span_stride, span_len, cache_dtype, tok_slot, tok_pos};
   // few rows (decoding): the heads of a token are spread over workgroups of four; many rows: a workgroup per token
   hipLaunchKernelGGL(qkv_prep_append_kernel, dim3(T, T >= 256 ? 1 : (H + G + 3) / 4), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), a);
@@ -438,9 +486,10 @@ int dihip_qkv_prep_append(void* stream, float* qkv, long ld, int q_off, int k_of
 
 static int gqa_check(const char* what, const float* out, long ldo, const float* q, long ldq, void* const* kspans, void* const* vspans,
                      int span_stride, int span_len, const void* sink, int w_dtype, int sink_mode, const float* gate, long ldg, int H, int G,
-                     int D, int DV) {
+                     int D, int DV, int maps, int keep_first) {
+  DIHIP_REQUIRE(maps >= 1 && maps <= 8 && keep_first >= 0, DIHIP_PARAM_ERROR, "%s: 1 to 8 maps per head, no negative count of kept keys", what);
   DIHIP_REQUIRE(out && q && kspans && vspans && span_stride > 0 && span_len > 0 && H > 0 && G > 0 && H % G == 0 && D > 0 && DV > 0 &&
-                    ldo >= (long)H * DV && ldq >= (long)H * D && seq_dtype_ok(w_dtype), DIHIP_PARAM_ERROR, "%s: bad argument", what);
+                    ldo >= (long)H * maps * DV && ldq >= (long)H * maps * D && seq_dtype_ok(w_dtype), DIHIP_PARAM_ERROR, "%s: bad argument", what);
   DIHIP_REQUIRE(sink_mode >= 0 && sink_mode <= 2 && (sink_mode != 1 || sink) && (!gate || ldg >= H), DIHIP_PARAM_ERROR,
                 "%s: bad sink mode or gate", what);
   return DIHIP_SUCCESS;
@@ -449,13 +498,13 @@ static int gqa_check(const char* what, const float* out, long ldo, const float* 
 int dihip_gqa_attn(void* stream, float* out, long ldo, const float* q, long ldq, void* const* kspans, void* const* vspans,
                    int span_stride, int span_len, int cache_dtype, const void* sink, int w_dtype, int sink_mode, float softcap,
                    const float* gate, long ldg, const int32_t* tok_slot, const int32_t* tok_pos, int T, int H, int G, int D, int DV,
-                   float scale) {
-  if (int rc = gqa_check("gqa_attn", out, ldo, q, ldq, kspans, vspans, span_stride, span_len, sink, w_dtype, sink_mode, gate, ldg, H, G, D, DV)) return rc;
+                   float scale, int maps, int window, int keep_first) {
+  if (int rc = gqa_check("gqa_attn", out, ldo, q, ldq, kspans, vspans, span_stride, span_len, sink, w_dtype, sink_mode, gate, ldg, H, G, D, DV, maps, keep_first)) return rc;
   DIHIP_REQUIRE(T >= 0 && tok_slot && tok_pos && seq_dtype_ok(cache_dtype), DIHIP_PARAM_ERROR, "gqa_attn: bad argument");
   DIHIP_REQUIRE(D <= 256 && DV <= 512, DIHIP_EXCEED_LIMIT_ERROR, "gqa_attn: head sizes above 256 (keys) / 512 (values)");
   if (T == 0) return DIHIP_SUCCESS;
   GqaArgs a{out, ldo, q, ldq, kspans, vspans, span_stride, span_len, sink, w_dtype, sink_mode, softcap, gate, ldg, tok_slot, tok_pos,
-            nullptr, nullptr, nullptr, H, G, D, DV, scale, nullptr, 0};
+            nullptr, nullptr, nullptr, H, G, D, DV, scale, nullptr, 0, maps, window, keep_first};
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   auto go = [&](auto ct, auto rv) {
     constexpr int CT = decltype(ct)::value, RV = decltype(rv)::value;
@@ -476,30 +525,31 @@ int dihip_gqa_attn_mc_supported(int D, int DV, int span_len, int cache_dtype) {
   return cache_dtype == DIHIP_BF16 && D % 8 == 0 && DV % 8 == 0 && D >= 8 && DV >= 8 && D <= 256 && DV <= 128 && span_len % 32 == 0;
 }
 
-size_t dihip_gqa_attn_mc_workspace_bytes(int T, int H, int DV, int nsplit) {
-  return nsplit > 1 ? (size_t)nsplit * T * H * (((DV + 15) & ~15) + 4) * sizeof(float) : 0;
+size_t dihip_gqa_attn_mc_workspace_bytes(int T, int HQ, int DV, int nsplit) {
+  return nsplit > 1 ? (size_t)nsplit * T * HQ * (((DV + 15) & ~15) + 4) * sizeof(float) : 0;
 }
 
 int dihip_gqa_attn_mc(void* stream, float* out, long ldo, const float* q, long ldq, void* const* kspans, void* const* vspans,
                       int span_stride, int span_len, const void* sink, int w_dtype, int sink_mode, float softcap, const float* gate,
                       long ldg, const int32_t* tok_pos, const int32_t* ent_slot, const int32_t* ent_row0, const int32_t* ent_count, int E,
-                      int max_count, int T, int H, int G, int D, int DV, float scale, int nsplit, void* ws, size_t ws_bytes) {
-  if (int rc = gqa_check("gqa_attn_mc", out, ldo, q, ldq, kspans, vspans, span_stride, span_len, sink, w_dtype, sink_mode, gate, ldg, H, G, D, DV)) return rc;
+                      int max_count, int T, int H, int G, int D, int DV, float scale, int maps, int window, int keep_first, int nsplit,
+                      void* ws, size_t ws_bytes) {
+  if (int rc = gqa_check("gqa_attn_mc", out, ldo, q, ldq, kspans, vspans, span_stride, span_len, sink, w_dtype, sink_mode, gate, ldg, H, G, D, DV, maps, keep_first)) return rc;
   DIHIP_REQUIRE(dihip_gqa_attn_mc_supported(D, DV, span_len, DIHIP_BF16), DIHIP_PARAM_ERROR,
                 "gqa_attn_mc: head sizes %d / %d (multiples of 8 up to 256 / 128) or span_len %d (a multiple of 32) not served", D, DV, span_len);
   DIHIP_REQUIRE(E >= 0 && T >= 0 && max_count >= 0 && tok_pos && ent_slot && ent_row0 && ent_count && ldo % 4 == 0 && ldq % 4 == 0,
                 DIHIP_PARAM_ERROR, "gqa_attn_mc: bad argument");
   DIHIP_REQUIRE((reinterpret_cast<uintptr_t>(out) & 15u) == 0 && (reinterpret_cast<uintptr_t>(q) & 15u) == 0, DIHIP_PARAM_ERROR,
                 "gqa_attn_mc: q / out must be 16-byte aligned");
-  DIHIP_REQUIRE(nsplit >= 1 && nsplit <= 1024 && (long)E * G <= 65535, DIHIP_PARAM_ERROR, "gqa_attn_mc: bad split / portion count");
-  DIHIP_REQUIRE(ws_bytes >= dihip_gqa_attn_mc_workspace_bytes(T, H, DV, nsplit) && (nsplit == 1 || ws), DIHIP_PARAM_ERROR,
+  DIHIP_REQUIRE(nsplit >= 1 && nsplit <= 1024 && (long)E * G * maps <= 65535, DIHIP_PARAM_ERROR, "gqa_attn_mc: bad split / portion count");
+  DIHIP_REQUIRE(ws_bytes >= dihip_gqa_attn_mc_workspace_bytes(T, H * maps, DV, nsplit) && (nsplit == 1 || ws), DIHIP_PARAM_ERROR,
                 "gqa_attn_mc: workspace too small");
   if (E == 0 || max_count == 0) return DIHIP_SUCCESS;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   GqaArgs a{out, ldo, q, ldq, kspans, vspans, span_stride, span_len, sink, w_dtype, sink_mode, softcap, gate, ldg, nullptr, tok_pos,
-            ent_slot, ent_row0, ent_count, H, G, D, DV, scale, (float*)ws, T * H};
+            ent_slot, ent_row0, ent_count, H, G, D, DV, scale, (float*)ws, T * H * maps, maps, window, keep_first};
   const int hpg = H / G, Dp = (D + 31) & ~31, Vp = (DV + 15) & ~15;
-  const dim3 grid((unsigned)(((long)max_count * hpg + 63) / 64), E * G, nsplit);
+  const dim3 grid((unsigned)(((long)max_count * hpg + 63) / 64), E * G * maps, nsplit);
   const size_t lds = (size_t)32 * ((Dp + 8) + (Vp + 8)) * 2;
   auto go = [&](auto dm, auto vm) {
     constexpr int DM = decltype(dm)::value, VM = decltype(vm)::value;
@@ -512,7 +562,19 @@ int dihip_gqa_attn_mc(void* stream, float* out, long ldo, const float* q, long l
   if (D <= 64) by_v(std::integral_constant<int, 64>{});
   else if (D <= 128) by_v(std::integral_constant<int, 128>{});
   else by_v(std::integral_constant<int, 256>{});
-  if (nsplit > 1) hipLaunchKernelGGL(gqa_attn_merge_kernel, dim3(T * H), dim3(256), 0, s, out, ldo, (const float*)ws, nsplit, T * H, H, DV, Vp, gate, ldg);
+  if (nsplit > 1) hipLaunchKernelGGL(gqa_attn_merge_kernel, dim3(T * H * maps), dim3(256), 0, s, out, ldo, (const float*)ws, nsplit, T * H * maps, H, maps, DV, Vp, gate, ldg);
+  return launch_status();
+}
+
+int dihip_maps_diff_norm(void* stream, void* y, int y_dtype, long ldy, const float* x, long ldx, float lam, float out_scale, float eps, int T,
+                         int H, int DV) {
+  DIHIP_REQUIRE(T >= 0 && H > 0 && DV > 0 && y && x && ldy >= (long)H * DV && ldx >= (long)H * 2 * DV && seq_dtype_ok(y_dtype), DIHIP_PARAM_ERROR,
+                "maps_diff_norm: bad argument");
+  DIHIP_REQUIRE(DV <= 512, DIHIP_EXCEED_LIMIT_ERROR, "maps_diff_norm: heads of more than 512 values");
+  if (T == 0) return DIHIP_SUCCESS;
+  const long pairs = (long)T * H;
+  hipLaunchKernelGGL(maps_diff_norm_kernel, dim3((unsigned)((pairs + 3) / 4)), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), y, y_dtype, ldy,
+                     x, ldx, lam, out_scale, eps, (int)pairs, H, DV);
   return launch_status();
 }
 

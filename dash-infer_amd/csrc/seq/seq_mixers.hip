@@ -25,6 +25,16 @@ __global__ __launch_bounds__(256) void embed_sum_kernel(float* __restrict__ h, c
   }
 }
 
+// columns [col0, col0 + K) of the table rows ids[t], times a constant, into rows of any stride and type
+template <int WT>
+__global__ __launch_bounds__(256) void embed_rows_kernel(void* __restrict__ y, int ydt, long ldy, const int32_t* __restrict__ ids,
+                                                         const void* __restrict__ table, long ldt, long col0, float scale, int K) {
+  const int t = blockIdx.x;
+  const size_t r = (size_t)ids[t] * ldt + col0;
+#pragma unroll 4
+  for (int k = threadIdx.x; k < K; k += 256) st_any(y, (size_t)t * ldy + k, ydt, load_ft<WT>(table, r + k) * scale);
+}
+
 // ------------------------------------------------------------------------------------------------ norms
 // sum of squares of a row, k ascending per thread, one fixed tree over the block
 __device__ __forceinline__ float row_sumsq(const float* __restrict__ x, int K, float* red) {
@@ -51,13 +61,51 @@ __device__ __forceinline__ float row_sumsq(const float* __restrict__ x, int K, f
 template <int WT>
 __global__ __launch_bounds__(256) void rmsnorm_strided_kernel(void* __restrict__ y, int ydt, long ldy, const float* __restrict__ x, long ldx,
                                                               const int32_t* __restrict__ row_idx, const void* __restrict__ gamma,
-                                                              float eps, int K) {
+                                                              float gamma_add, float out_scale, float eps, int K) {
   __shared__ float red[4];
   const int i = blockIdx.x;
   const float* xr = x + (size_t)(row_idx ? row_idx[i] : i) * ldx;
   const float inv = 1.f / sqrtf(row_sumsq(xr, K, red) / (float)K + eps);
+  if (gamma_add == 0.f && out_scale == 1.f) {
 #pragma unroll 4
-  for (int k = threadIdx.x; k < K; k += 256) st_any(y, (size_t)i * ldy + k, ydt, xr[k] * inv * load_ft<WT>(gamma, k));
+    for (int k = threadIdx.x; k < K; k += 256) st_any(y, (size_t)i * ldy + k, ydt, xr[k] * inv * load_ft<WT>(gamma, k));
+  } else {
+#pragma unroll 4
+    for (int k = threadIdx.x; k < K; k += 256) st_any(y, (size_t)i * ldy + k, ydt, xr[k] * inv * (gamma_add + load_ft<WT>(gamma, k)) * out_scale);
+  }
+}
+
+// The residual step of a layer with norms before AND after its sublayers, one workgroup per row:
+//   xo = x_in + m / rms(m) * (add_m + gamma_m)   (m NULL: xo = x_in);   x_out = xo;   xc = xo (any type / stride);
+//   h  = xo / rms(xo) * (add_h + gamma_h)        (the next sublayer's input norm)
+// Every thread re-reads only what it wrote itself.
+template <int WT>
+__global__ __launch_bounds__(256) void residual_norm_step_kernel(float* x_out, const float* x_in, const float* __restrict__ m, long ldm,
+                                                                 const void* __restrict__ gamma_m, float add_m, const void* __restrict__ gamma_h,
+                                                                 float add_h, float eps, void* __restrict__ xc, int cdt, long ldc,
+                                                                 void* __restrict__ h, int hdt, long ldh, int K) {
+  __shared__ float red[4];
+  const int t = blockIdx.x;
+  const size_t row = (size_t)t * K;
+  const float* mr = m ? m + (size_t)t * ldm : nullptr;
+  float inv_m = 0.f;
+  if (m) inv_m = 1.f / sqrtf(row_sumsq(mr, K, red) / (float)K + eps);
+  float ss = 0.f;
+#pragma unroll 4
+  for (int k = threadIdx.x; k < K; k += 256) {
+    float xo = x_in[row + k];
+    if (m) {
+      xo += mr[k] * inv_m * (add_m + load_ft<WT>(gamma_m, k));
+      x_out[row + k] = xo;
+    }
+    if (xc) st_any(xc, (size_t)t * ldc + k, cdt, xo);
+    ss = __builtin_fmaf(xo, xo, ss);
+  }
+  if (!h) return;
+  const float inv = 1.f / sqrtf(block256_sum(ss, red) / (float)K + eps);
+  const float* src = m ? x_out : x_in;
+#pragma unroll 4
+  for (int k = threadIdx.x; k < K; k += 256) st_any(h, (size_t)t * ldh + k, hdt, src[row + k] * inv * (add_h + load_ft<WT>(gamma_h, k)));
 }
 
 template <int WT>
@@ -399,13 +447,36 @@ int dihip_embed_sum(void* stream, float* h, const int32_t* ids, const void* tabl
   return launch_status();
 }
 
+int dihip_embed_rows(void* stream, void* y, int y_dtype, long ldy, const int32_t* ids, const void* table, int w_dtype, long ldt, long col0,
+                     float scale, int T, int K) {
+  DIHIP_REQUIRE(T >= 0 && K > 0 && y && ids && table && ldy >= K && col0 >= 0 && ldt >= col0 + K && seq_dtype_ok(w_dtype) && seq_dtype_ok(y_dtype),
+                DIHIP_PARAM_ERROR, "embed_rows: bad argument");
+  if (T == 0) return DIHIP_SUCCESS;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  if (w_dtype == DIHIP_F32) hipLaunchKernelGGL(embed_rows_kernel<DIHIP_F32>, dim3(T), dim3(256), 0, s, y, y_dtype, ldy, ids, table, ldt, col0, scale, K);
+  else hipLaunchKernelGGL(embed_rows_kernel<DIHIP_BF16>, dim3(T), dim3(256), 0, s, y, y_dtype, ldy, ids, table, ldt, col0, scale, K);
+  return launch_status();
+}
+
+int dihip_residual_norm_step(void* stream, float* x_out, const float* x_in, const float* m, long ldm, const void* gamma_m, float add_m,
+                             const void* gamma_h, float add_h, int w_dtype, float eps, void* xc, int xc_dtype, long ldc, void* h, int h_dtype,
+                             long ldh, int T, int K) {
+  DIHIP_REQUIRE(T >= 0 && K > 0 && x_in && (!m || (x_out && gamma_m && ldm >= K)) && (!h || (gamma_h && ldh >= K)) && (!xc || ldc >= K) &&
+                    seq_dtype_ok(w_dtype) && seq_dtype_ok(xc_dtype) && seq_dtype_ok(h_dtype), DIHIP_PARAM_ERROR, "residual_norm_step: bad argument");
+  if (T == 0) return DIHIP_SUCCESS;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  if (w_dtype == DIHIP_F32) hipLaunchKernelGGL(residual_norm_step_kernel<DIHIP_F32>, dim3(T), dim3(256), 0, s, x_out, x_in, m, ldm, gamma_m, add_m, gamma_h, add_h, eps, xc, xc_dtype, ldc, h, h_dtype, ldh, K);
+  else hipLaunchKernelGGL(residual_norm_step_kernel<DIHIP_BF16>, dim3(T), dim3(256), 0, s, x_out, x_in, m, ldm, gamma_m, add_m, gamma_h, add_h, eps, xc, xc_dtype, ldc, h, h_dtype, ldh, K);
+  return launch_status();
+}
+
 int dihip_rmsnorm_strided(void* stream, void* y, int y_dtype, long ldy, const float* x, long ldx, const int32_t* row_idx,
-                          const void* gamma, int w_dtype, float eps, int M, int K) {
+                          const void* gamma, int w_dtype, float gamma_add, float out_scale, float eps, int M, int K) {
   DIHIP_REQUIRE(M >= 0 && K > 0 && y && x && gamma && ldy >= K && ldx >= K && seq_dtype_ok(y_dtype) && seq_dtype_ok(w_dtype),
                 DIHIP_PARAM_ERROR, "rmsnorm_strided: bad argument");
   if (M == 0) return DIHIP_SUCCESS;
-  if (w_dtype == DIHIP_F32) hipLaunchKernelGGL(rmsnorm_strided_kernel<DIHIP_F32>, dim3(M), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), y, y_dtype, ldy, x, ldx, row_idx, gamma, eps, K);
-  else hipLaunchKernelGGL(rmsnorm_strided_kernel<DIHIP_BF16>, dim3(M), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), y, y_dtype, ldy, x, ldx, row_idx, gamma, eps, K);
+  if (w_dtype == DIHIP_F32) hipLaunchKernelGGL(rmsnorm_strided_kernel<DIHIP_F32>, dim3(M), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), y, y_dtype, ldy, x, ldx, row_idx, gamma, gamma_add, out_scale, eps, K);
+  else hipLaunchKernelGGL(rmsnorm_strided_kernel<DIHIP_BF16>, dim3(M), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), y, y_dtype, ldy, x, ldx, row_idx, gamma, gamma_add, out_scale, eps, K);
   return launch_status();
 }
 

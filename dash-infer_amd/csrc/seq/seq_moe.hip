@@ -1,14 +1,47 @@
 // seq_moe.hip -- routing and glue of the mixture-of-experts feed-forward (the expert products are dihip_linear_segmented):
-//   moe_route      per token: the `top` experts of largest router logit (ties: the lower index), weights = softmax over the
-//                  chosen logits alone, f32
+//   moe_route      per token, f32: the `top` experts of largest router logit (ties: the lower index), weights = softmax over the
+//                  chosen logits alone; or (scoring 1) scores = softmax over ALL logits, the choice by score + a correction per
+//                  expert, weights = the chosen scores over their sum
 //   moe_sort       the (token, choice) pairs grouped by expert in a fixed order: segment bounds per expert, the token each
 //                  sorted row reads, and where each pair went
-//   moe_glu        the experts' activation on [gate | up] rows
-//   moe_combine    out[t] = sum over the token's choices, in order, of weight * the expert's output row
+//   moe_glu        the experts' activation on [gate | up] rows (clamped sigmoid unit, or silu(gate) * up)
+//   moe_combine    out[t] = sum over the token's choices, in order, of weight * the expert's output row -- the token's own input
+//                  row for the experts past the real ones (identity experts) -- plus an optional row added for every token
 #include "seq_common.h"
 
 namespace dihip {
 namespace {
+
+// scoring 1: every logit is read three times (maximum, denominator, choice): E is small and the row stays in cache
+__global__ __launch_bounds__(256) void moe_route_scores_kernel(const float* __restrict__ logits, long ldl, const void* __restrict__ corr, int cdt,
+                                                               int32_t* __restrict__ ids, float* __restrict__ wts, int T, int E, int top) {
+  const int t = blockIdx.x * 256 + threadIdx.x;
+  if (t >= T) return;
+  const float* z = logits + (size_t)t * ldl;
+  float zmax = -INFINITY, den = 0.f;
+  for (int e = 0; e < E; ++e) zmax = fmaxf(zmax, z[e]);
+  for (int e = 0; e < E; ++e) den += expf(z[e] - zmax);
+  float best[32];
+  int bi[32];
+  float sum = 0.f;
+  for (int k = 0; k < top; ++k) {
+    float bv = -INFINITY, bs = 0.f;
+    int bx = -1;
+    for (int e = 0; e < E; ++e) {
+      bool used = false;
+      for (int j = 0; j < k; ++j) used |= bi[j] == e;
+      const float sc = expf(z[e] - zmax) / den;
+      const float v = sc + (corr ? ld_any(corr, e, cdt) : 0.f);
+      if (!used && (bx < 0 || v > bv)) { bv = v; bx = e; bs = sc; }
+    }
+    best[k] = bs; bi[k] = bx;
+    sum += bs;
+  }
+  for (int k = 0; k < top; ++k) {
+    ids[(size_t)t * top + k] = bi[k];
+    wts[(size_t)t * top + k] = best[k] / (sum + 1e-20f);
+  }
+}
 
 __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits, long ldl, int32_t* __restrict__ ids,
                                                         float* __restrict__ wts, int T, int E, int top) {
@@ -77,9 +110,14 @@ __global__ __launch_bounds__(256) void moe_place_kernel(const int32_t* __restric
 }
 
 __global__ __launch_bounds__(256) void moe_glu_kernel(void* __restrict__ y, int ydt, long ldy, const float* __restrict__ gu, long ldgu, int F,
-                                                      float limit, float slope) {
+                                                      float limit, float slope, int unit) {
   const int r = blockIdx.x;
   for (int c = blockIdx.y * 256 + threadIdx.x; c < F; c += 256 * gridDim.y) {
+    if (unit == 1) {      // silu(gate) * up
+      const float g = gu[(size_t)r * ldgu + c], u = gu[(size_t)r * ldgu + F + c];
+      st_any(y, (size_t)r * ldy + c, ydt, g / (1.f + expf(-g)) * u);
+      continue;
+    }
     const float g = fminf(gu[(size_t)r * ldgu + c], limit);
     const float u = fminf(fmaxf(gu[(size_t)r * ldgu + F + c], -limit), limit);
     st_any(y, (size_t)r * ldy + c, ydt, g * (1.f / (1.f + expf(-slope * g))) * (u + 1.f));
@@ -87,11 +125,18 @@ __global__ __launch_bounds__(256) void moe_glu_kernel(void* __restrict__ y, int 
 }
 
 __global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ out, long ldo, const float* __restrict__ rows, long ldr,
-                                                          const int32_t* __restrict__ dst, const float* __restrict__ wts, int top, int K) {
+                                                          const int32_t* __restrict__ dst, const float* __restrict__ wts, int top, int K,
+                                                          const int32_t* __restrict__ ids, int n_real, const void* __restrict__ own, int odt,
+                                                          long ldown, const float* __restrict__ add, long ldadd) {
   const int t = blockIdx.x;
   for (int c = blockIdx.y * 256 + threadIdx.x; c < K; c += 256 * gridDim.y) {
     float acc = 0.f;
-    for (int k = 0; k < top; ++k) acc = __builtin_fmaf(wts[(size_t)t * top + k], rows[(size_t)dst[(size_t)t * top + k] * ldr + c], acc);
+    for (int k = 0; k < top; ++k) {
+      const size_t pr = (size_t)t * top + k;
+      const float v = ids && ids[pr] >= n_real ? ld_any(own, (size_t)t * ldown + c, odt) : rows[(size_t)dst[pr] * ldr + c];
+      acc = __builtin_fmaf(wts[pr], v, acc);
+    }
+    if (add) acc += add[(size_t)t * ldadd + c];
     out[(size_t)t * ldo + c] = acc;
   }
 }
@@ -104,29 +149,34 @@ using namespace dihip;
 extern "C" {
 
 int dihip_seq_moe_route(void* stream, const float* logits, long ldl, int32_t* ids, float* wts, int32_t* counts, int32_t* seg, int32_t* src_row,
-                    int32_t* dst, int T, int E, int top) {
+                    int32_t* dst, int T, int E, int top, int scoring, const void* correction, int w_dtype) {
+  DIHIP_REQUIRE((scoring == 0 || scoring == 1) && (!correction || scoring == 1) && seq_dtype_ok(w_dtype), DIHIP_PARAM_ERROR,
+                "moe_route: unknown scoring (a correction goes with scoring 1)");
   DIHIP_REQUIRE(T >= 0 && E > 0 && top > 0 && top <= E && top <= 32 && E <= 65535 && logits && ids && wts && counts && seg && src_row && dst &&
                     ldl >= E, DIHIP_PARAM_ERROR, "moe_route: bad argument (at most 32 choices per token)");
   if (T == 0) return DIHIP_SUCCESS;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-  hipLaunchKernelGGL(moe_route_kernel, dim3((T + 255) / 256), dim3(256), 0, s, logits, ldl, ids, wts, T, E, top);
+  if (scoring == 1) hipLaunchKernelGGL(moe_route_scores_kernel, dim3((T + 255) / 256), dim3(256), 0, s, logits, ldl, correction, w_dtype, ids, wts, T, E, top);
+  else hipLaunchKernelGGL(moe_route_kernel, dim3((T + 255) / 256), dim3(256), 0, s, logits, ldl, ids, wts, T, E, top);
   hipLaunchKernelGGL(moe_count_kernel, dim3(E), dim3(256), 0, s, ids, T * top, counts);
   hipLaunchKernelGGL(moe_place_kernel, dim3(E), dim3(256), 0, s, ids, T * top, top, E, counts, seg, src_row, dst);
   return launch_status();
 }
 
-int dihip_seq_moe_glu(void* stream, void* y, int y_dtype, long ldy, const float* gu, long ldgu, int R, int F, float limit, float slope) {
-  DIHIP_REQUIRE(R >= 0 && F > 0 && y && gu && ldy >= F && ldgu >= 2 * (long)F && seq_dtype_ok(y_dtype), DIHIP_PARAM_ERROR, "moe_glu: bad argument");
+int dihip_seq_moe_glu(void* stream, void* y, int y_dtype, long ldy, const float* gu, long ldgu, int R, int F, float limit, float slope, int unit) {
+  DIHIP_REQUIRE((unit == 0 || unit == 1) && R >= 0 && F > 0 && y && gu && ldy >= F && ldgu >= 2 * (long)F && seq_dtype_ok(y_dtype), DIHIP_PARAM_ERROR, "moe_glu: bad argument");
   if (R == 0) return DIHIP_SUCCESS;
-  hipLaunchKernelGGL(moe_glu_kernel, dim3(R, R >= 256 ? 1 : (F + 1023) / 1024), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), y, y_dtype, ldy, gu, ldgu, F, limit, slope);
+  hipLaunchKernelGGL(moe_glu_kernel, dim3(R, R >= 256 ? 1 : (F + 1023) / 1024), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), y, y_dtype, ldy, gu, ldgu, F, limit, slope, unit);
   return launch_status();
 }
 
 int dihip_seq_moe_combine(void* stream, float* out, long ldo, const float* rows, long ldr, const int32_t* dst, const float* wts, int T, int top,
-                      int K) {
+                      int K, const int32_t* ids, int n_real, const void* own, int own_dtype, long ldown, const float* add, long ldadd) {
   DIHIP_REQUIRE(T >= 0 && top > 0 && K > 0 && out && rows && dst && wts && ldo >= K && ldr >= K, DIHIP_PARAM_ERROR, "moe_combine: bad argument");
+  DIHIP_REQUIRE((!ids || (own && ldown >= K && seq_dtype_ok(own_dtype) && n_real >= 0)) && (!add || ldadd >= K), DIHIP_PARAM_ERROR,
+                "moe_combine: identity experts need the tokens' own rows; added rows at least K wide");
   if (T == 0) return DIHIP_SUCCESS;
-  hipLaunchKernelGGL(moe_combine_kernel, dim3(T, T >= 256 ? 1 : (K + 1023) / 1024), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), out, ldo, rows, ldr, dst, wts, top, K);
+  hipLaunchKernelGGL(moe_combine_kernel, dim3(T, T >= 256 ? 1 : (K + 1023) / 1024), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), out, ldo, rows, ldr, dst, wts, top, K, ids, n_real, own, own_dtype, ldown, add, ldadd);
   return launch_status();
 }
 

@@ -10,11 +10,15 @@ to rows of the same shape, reading and updating what its sequences left in the s
   GroupedQueryAttention  causal attention over paged key and value caches with fewer key/value heads than query heads; options:
                          unit-RMS norm of queries and keys, rotary positions (paired or half-split layout, part of the head,
                          frequencies rescaled for longer contexts), biases, a sink logit (per head or the constant 0), a tanh cap
-                         on the scores, a sigmoid gate per head, values mixed with those of an earlier layer of the same step
+                         on the scores, a sigmoid gate per head, values mixed with those of an earlier layer of the same step,
+                         a sliding window that keeps the first keys of the sequence, two softmax maps per head whose difference
+                         is normed per head (differential attention), several runs per step with a cache each (looped layers)
   GatedLinearAttention   linear attention with a decay per key channel and a matrix state per head (f32, per slot), unit-RMS
                          norm per head, silu output gate
   GatedMlp               down(act(gate(h)) * up(h))
-  ExpertMlp              top-k routed experts with clamped gated units, weights = softmax over the chosen logits
+  ExpertMlp              top-k routed experts; units: clamped sigmoid-gated or silu-gated; routing: softmax over the chosen logits,
+                         or softmax scores over all router outputs with a correction added for the choice alone; router outputs
+                         past the real experts stand for identity experts; an always-on shared expert
 Matrix products run in ctx.math (seq_ops.MATH_F32 / MATH_BF16); norms, scores, gates of the recurrence, decays and
 state are f32 in both.
 """
@@ -145,13 +149,21 @@ class GroupedQueryAttention:
     LAYOUTS = {"pairs": 0, "halves": 1}
 
     def __init__(self, key, heads, kv_heads, dim, vdim, scale, w, state, cache_dtype, rot_dims=0, rot_base=10000.0, rot_layout="pairs",
-                 rot_scaling=None, qk_norm=False, sink=None, softcap=None, head_gate=False, value_mix=None):
-        """w: q [heads*dim, width], k [kv_heads*dim, width], v [kv_heads*vdim, width] (+ q.b / k.b / v.b where present), q.norm /
-        k.norm [dim] (qk_norm), g [heads, width] (head_gate), o [width, heads*vdim].  sink: None, "zero" or a tensor [heads].
-        value_mix: None, ("source", name): this layer's values are kept under `name` for the step, or ("mix", name, lam):
-        v <- (1 - lam) v + lam * the values kept under `name`."""
+                 rot_scaling=None, qk_norm=False, sink=None, softcap=None, head_gate=False, value_mix=None, window=0, keep_first=0,
+                 differential=None, runs=1):
+        """w: q [heads*maps*dim, width], k [kv_heads*maps*dim, width], v [kv_heads*vdim, width] (+ q.b / k.b / v.b / o.b where
+        present), q.norm / k.norm [dim] (qk_norm), g [heads, width] (head_gate), o [width, heads*vdim].  sink: None, "zero" or a
+        tensor [heads].  value_mix: None, ("source", name): this layer's values are kept under `name` for the step, or
+        ("mix", name, lam): v <- (1 - lam) v + lam * the values kept under `name`.
+        window > 0: a row reads the keys less than `window` positions back and the first keep_first keys of its sequence.
+        differential: None (maps = 1), or (lam, out_scale): two softmax maps per head (their queries and keys side by side in q
+        and k) over the same values, out = unit_rms(first - lam * second) * out_scale per head.
+        runs: how often the layer runs in a step (a looped layer); every run has key and value caches of its own."""
         assert heads % kv_heads == 0
         self.H, self.G, self.D, self.V, self.scale = heads, kv_heads, dim, vdim, float(scale)
+        self.maps, self.differential = (2, (float(differential[0]), float(differential[1]))) if differential is not None else (1, None)
+        self.window, self.keep_first = int(window or 0), int(keep_first or 0)
+        heads, kv_heads = heads * self.maps, kv_heads * self.maps     # query / key vectors per token from here on
         dev = w["q"].device
         parts = [w["q"], w["k"], w["v"]] + ([w["g"]] if head_gate else [])
         n = sum(p.shape[0] for p in parts)
@@ -159,14 +171,14 @@ class GroupedQueryAttention:
             parts.append(torch.zeros(4 - n % 4, w["q"].shape[1], dtype=w["q"].dtype, device=dev))
         self.w_in = torch.cat(parts, 0).contiguous()
         self.k_lo, self.v_lo = heads * dim, (heads + kv_heads) * dim
-        self.g_lo = self.v_lo + kv_heads * vdim
+        self.g_lo = self.v_lo + self.G * vdim
         self.n_in = self.w_in.shape[0]
         self.head_gate = head_gate
         self.b_in = None
         if "q.b" in w or "k.b" in w or "v.b" in w:
             zero = lambda n: torch.zeros(n, dtype=self.w_in.dtype, device=dev)
-            b = [w.get("q.b", zero(heads * dim)), w.get("k.b", zero(kv_heads * dim)), w.get("v.b", zero(kv_heads * vdim))]
-            b = torch.cat(b + ([zero(heads)] if head_gate else []), 0)
+            b = [w.get("q.b", zero(heads * dim)), w.get("k.b", zero(kv_heads * dim)), w.get("v.b", zero(self.G * vdim))]
+            b = torch.cat(b + ([zero(self.H)] if head_gate else []), 0)
             self.b_in = torch.cat([b, zero(self.n_in - b.shape[0])], 0).contiguous()
         self.q_norm, self.k_norm = (w["q.norm"].contiguous(), w["k.norm"].contiguous()) if qk_norm else (None, None)
         self.rot_dims, self.layout = int(rot_dims), self.LAYOUTS[rot_layout]
@@ -183,14 +195,18 @@ class GroupedQueryAttention:
             self.sink_mode, self.sink = so.SINK_PER_HEAD, sink.contiguous()
         self.softcap = float(softcap or 0.0)
         self.value_mix = value_mix
-        self.o = w["o"].contiguous()
-        assert self.o.shape[1] == heads * vdim and w["q"].shape[0] == heads * dim and w["k"].shape[0] == kv_heads * dim
-        self.ktable = state.add_span_cache(key + ".k", kv_heads * dim, cache_dtype)
-        self.vtable = state.add_span_cache(key + ".v", kv_heads * vdim, cache_dtype)
-        self.mc = so.gqa_attn_mc_supported(self.ktable, self.vtable, kv_heads) and self.n_in % 4 == 0 and (heads * dim) % 4 == 0
+        self.o, self.o_b = w["o"].contiguous(), w.get("o.b")
+        assert self.o.shape[1] == self.H * vdim and w["q"].shape[0] == heads * dim and w["k"].shape[0] == kv_heads * dim
+        assert w["v"].shape[0] == self.G * vdim
+        names = [key] if runs == 1 else [f"{key}.run{r}" for r in range(runs)]
+        self.ktables = [state.add_span_cache(n + ".k", kv_heads * dim, cache_dtype) for n in names]
+        self.vtables = [state.add_span_cache(n + ".v", self.G * vdim, cache_dtype) for n in names]
+        self.ktable, self.vtable = self.ktables[0], self.vtables[0]
+        self.mc = so.gqa_attn_mc_supported(dim, vdim, self.ktable) and self.n_in % 4 == 0 and (heads * dim) % 4 == 0
 
-    def __call__(self, ctx, h, h16=None):
+    def __call__(self, ctx, h, h16=None, run=0):
         H, G, D, V = self.H, self.G, self.D, self.V
+        ktable, vtable = self.ktables[run], self.vtables[run]
         a = so.linear(h16 if h16 is not None else h, self.w_in, self.b_in, act="sigmoid" if self.head_gate else None,
                       act_cols=(self.g_lo, self.n_in), math=ctx.math)                                        # [q | k | v | gate]
         vin = vout = None
@@ -202,15 +218,18 @@ class GroupedQueryAttention:
                 vin, lam = ctx.shared[self.value_mix[1]], self.value_mix[2]
                 assert vin.shape[1] == G * V, "mixed values must have this layer's shape"
         so.qkv_prep_append(a, 0, self.k_lo, self.v_lo, H, G, D, V, self.q_norm, self.k_norm, ctx.eps, self.freq, self.rot_dims, self.layout,
-                           self.mag, lam, vin, vout, self.ktable, self.vtable, ctx.tok_slot, ctx.tok_pos)
+                           self.mag, lam, vin, vout, ktable, vtable, ctx.tok_slot, ctx.tok_pos, maps=self.maps)
         gate = a[:, self.g_lo:] if self.head_gate else None
         if ctx.math == so.MATH_BF16 and self.mc:
-            o = so.gqa_attn_mc(a, self.ktable, self.vtable, ctx.tok_pos, ctx.ent_slot, ctx.ent_row0, ctx.ent_count, ctx.max_count, ctx.max_pos,
-                               H, G, D, V, self.scale, self.sink, self.sink_mode, self.softcap, gate)
+            o = so.gqa_attn_mc(a, ktable, vtable, ctx.tok_pos, ctx.ent_slot, ctx.ent_row0, ctx.ent_count, ctx.max_count, ctx.max_pos,
+                               H, G, D, V, self.scale, self.sink, self.sink_mode, self.softcap, gate, maps=self.maps, window=self.window,
+                               keep_first=self.keep_first)
         else:
-            o = so.gqa_attn(a, self.ktable, self.vtable, ctx.tok_slot, ctx.tok_pos, H, G, D, V, self.scale, self.sink, self.sink_mode,
-                            self.softcap, gate)
-        return so.linear(o, self.o, math=ctx.math)
+            o = so.gqa_attn(a, ktable, vtable, ctx.tok_slot, ctx.tok_pos, H, G, D, V, self.scale, self.sink, self.sink_mode,
+                            self.softcap, gate, maps=self.maps, window=self.window, keep_first=self.keep_first)
+        if self.differential is not None:
+            o = so.maps_diff_norm(o, self.differential[0], self.differential[1], ctx.eps, H, V, out=ctx.act_buffer(H * V))
+        return so.linear(o, self.o, self.o_b, math=ctx.math)
 
 
 class GatedLinearAttention:
@@ -251,24 +270,37 @@ class GatedMlp:
 class ExpertMlp:
     GLU_SLOPE = 1.702    # g * sigmoid(1.702 g): the sigmoid form of gelu
 
-    def __init__(self, router, router_b, gates, ups, downs, top, limit):
-        """gates / ups [ff, width] and downs [width, ff] per expert; an expert is down(glu(min(gate h, limit), clamp(up h, +-limit)))"""
+    def __init__(self, router, router_b, gates, ups, downs, top, limit=0.0, unit="clamped", scoring="chosen_softmax", correction=None,
+                 identity=0, shared=None):
+        """gates / ups [ff, width] and downs [width, ff] per expert.  unit "clamped": an expert is
+        down(glu(min(gate h, limit), clamp(up h, +-limit))); "silu": down(silu(gate h) * (up h)).
+        scoring "chosen_softmax": the `top` largest router logits, weights = softmax over them alone; "scores": scores = softmax over
+        all router outputs, the choice by score + correction [experts + identity] (None: the score alone), weights = the chosen
+        scores over their sum.  identity: the last `identity` router outputs have no tensors: such an expert returns its input.
+        shared: a feed-forward (GatedMlp) that runs for every token and is added, or None."""
         self.E, self.top, self.limit = len(gates), int(top), float(limit)
-        self.router, self.router_b = router.contiguous(), router_b.contiguous()
+        self.unit = {"clamped": so.UNIT_CLAMPED, "silu": so.UNIT_SILU}[unit]
+        self.scoring = {"chosen_softmax": so.ROUTE_CHOSEN_SOFTMAX, "scores": so.ROUTE_SCORES}[scoring]
+        self.identity, self.shared = int(identity), shared
+        self.router, self.router_b = router.contiguous(), router_b.contiguous() if router_b is not None else None
+        self.correction = correction.contiguous() if correction is not None else None
         self.F = gates[0].shape[0]
         self.w_gu = torch.stack([torch.cat([g, u], 0) for g, u in zip(gates, ups)]).contiguous()    # [E, 2 ff, width]
         self.w_down = torch.stack(list(downs)).contiguous()                                          # [E, width, ff]
-        assert self.router.shape[0] == self.E and 0 < self.top <= self.E
+        assert self.router.shape[0] == self.E + self.identity and 0 < self.top <= self.E + self.identity
+        assert self.correction is None or (self.scoring == so.ROUTE_SCORES and self.correction.shape == (self.E + self.identity,))
 
     def __call__(self, ctx, h, h16=None):
         x = h16 if h16 is not None else h
         T, R = ctx.T, ctx.T * self.top
         logits = so.linear(x, self.router, self.router_b, math=so.MATH_F32 if ctx.math == so.MATH_F32 else so.MATH_F32_STREAM)
-        _, wts, seg, src_row, dst = so.moe_route(logits, self.top)
+        ids, wts, seg, src_row, dst = so.moe_route(logits, self.top, self.scoring, self.correction)
+        # the pairs of the identity experts sort behind those of the real ones: the expert products never see their rows
         gu = so.linear_segmented(x, self.w_gu, seg, src_row, T, R, math=ctx.math)
-        y = so.moe_glu(gu, self.F, self.limit, self.GLU_SLOPE, ctx_rows(ctx, R, self.F))
+        y = so.moe_glu(gu, self.F, self.limit, self.GLU_SLOPE, ctx_rows(ctx, R, self.F), unit=self.unit)
         d = so.linear_segmented(y, self.w_down, seg, None, T, R, math=ctx.math)
-        return so.moe_combine(d, dst, wts, T, self.top)
+        add = self.shared(ctx, h, h16) if self.shared is not None else None
+        return so.moe_combine(d, dst, wts, T, self.top, ids=ids if self.identity else None, n_real=self.E, own=x, add=add)
 
 
 def ctx_rows(ctx, rows, n):

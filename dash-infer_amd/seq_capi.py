@@ -22,7 +22,9 @@ _SIGS = {
     "dihip_seq_last_error": (C.c_char_p, []),
     "dihip_linear": (i32, [vp, vp, i32, lng, lng, i32, vp, i32, vp, vp, i32, lng, lng, vp, lng, i32, i32, i32, i32, i32, i32, i32, i32]),
     "dihip_embed_sum": (i32, [vp, vp, vp, vp, vp, vp, i32, i32, i32]),
-    "dihip_rmsnorm_strided": (i32, [vp, vp, i32, lng, vp, lng, vp, vp, i32, f32, i32, i32]),
+    "dihip_embed_rows": (i32, [vp, vp, i32, lng, vp, vp, i32, lng, lng, f32, i32, i32]),
+    "dihip_rmsnorm_strided": (i32, [vp, vp, i32, lng, vp, lng, vp, vp, i32, f32, f32, f32, i32, i32]),
+    "dihip_residual_norm_step": (i32, [vp, vp, vp, vp, lng, vp, f32, vp, f32, i32, f32, vp, i32, lng, vp, i32, lng, i32, i32]),
     "dihip_norm_span_append": (i32, [vp, vp, i32, i32, i32, vp, lng, vp, i32, f32, vp, vp, i32, i32]),
     "dihip_norm_residual_mix": (i32, [vp, vp, vp, vp, lng, vp, i32, f32, vp, sz, vp, i32, vp, vp, i32, i32]),
     "dihip_latent_window_attn": (i32, [vp, vp, lng, vp, lng, vp, i32, i32, i32, vp, i32, vp, vp, i32, i32, i32, i32, f32, i32]),
@@ -36,19 +38,21 @@ _SIGS = {
     "dihip_gated_recurrence_chunked": (i32, [vp, vp, lng, vp, vp, lng, vp, lng, vp, lng, vp, i32, f32, vp, vp, vp, vp, i32, i32, i32, vp, sz]),
     "dihip_linear_segmented": (i32, [vp, vp, i32, lng, vp, i32, vp, vp, i32, lng, i32, i32, i32, i32, vp, vp, i32, i32, i32]),
     "dihip_add_dyt": (i32, [vp, vp, vp, vp, lng, vp, lng, vp, f32, vp, vp, i32, vp, vp, i32, i32]),
-    "dihip_qkv_prep_append": (i32, [vp, vp, lng, i32, i32, i32, i32, i32, i32, i32, vp, vp, i32, f32, vp, i32, i32, f32, f32, vp, vp, lng, vp, vp,
+    "dihip_qkv_prep_append": (i32, [vp, vp, lng, i32, i32, i32, i32, i32, i32, i32, i32, vp, vp, i32, f32, vp, i32, i32, f32, f32, vp, vp, lng, vp, vp,
                                     i32, i32, i32, vp, vp, i32]),
-    "dihip_gqa_attn": (i32, [vp, vp, lng, vp, lng, vp, vp, i32, i32, i32, vp, i32, i32, f32, vp, lng, vp, vp, i32, i32, i32, i32, i32, f32]),
+    "dihip_gqa_attn": (i32, [vp, vp, lng, vp, lng, vp, vp, i32, i32, i32, vp, i32, i32, f32, vp, lng, vp, vp, i32, i32, i32, i32, i32, f32, i32, i32,
+                             i32]),
+    "dihip_maps_diff_norm": (i32, [vp, vp, i32, lng, vp, lng, f32, f32, f32, i32, i32, i32]),
     "dihip_gqa_attn_mc_supported": (i32, [i32, i32, i32, i32]),
     "dihip_gqa_attn_mc_workspace_bytes": (sz, [i32, i32, i32, i32]),
     "dihip_gqa_attn_mc": (i32, [vp, vp, lng, vp, lng, vp, vp, i32, i32, vp, i32, i32, f32, vp, lng, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32,
-                                i32, f32, i32, vp, sz]),
+                                i32, f32, i32, i32, i32, i32, vp, sz]),
     "dihip_gla_workspace_bytes": (sz, [i32, i32, i32, i32, i32, i32, i32]),
     "dihip_gla": (i32, [vp, vp, lng, vp, lng, vp, lng, vp, lng, vp, lng, f32, f32, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, vp, sz]),
     "dihip_head_rmsnorm_mul": (i32, [vp, vp, i32, lng, vp, lng, vp, i32, f32, vp, lng, i32, i32, i32]),
-    "dihip_seq_moe_route": (i32, [vp, vp, lng, vp, vp, vp, vp, vp, vp, i32, i32, i32]),
-    "dihip_seq_moe_glu": (i32, [vp, vp, i32, lng, vp, lng, i32, i32, f32, f32]),
-    "dihip_seq_moe_combine": (i32, [vp, vp, lng, vp, lng, vp, vp, i32, i32, i32]),
+    "dihip_seq_moe_route": (i32, [vp, vp, lng, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, vp, i32]),
+    "dihip_seq_moe_glu": (i32, [vp, vp, i32, lng, vp, lng, i32, i32, f32, f32, i32]),
+    "dihip_seq_moe_combine": (i32, [vp, vp, lng, vp, lng, vp, vp, i32, i32, i32, vp, i32, vp, i32, lng, vp, lng]),
     "dihip_gated_recurrence": (i32, [vp, vp, lng, vp, vp, lng, vp, lng, vp, lng, vp, i32, f32, vp, vp, vp, vp, i32, i32]),
 }
 

@@ -62,14 +62,45 @@ def embed_sum(ids, table, rows2=None, table2=None, out=None):
     return h
 
 
-def rmsnorm(x, gamma, eps, row_idx=None, out=None):
+def embed_rows(ids, table, col0=0, cols=None, scale=1.0, out=None):
+    """out[t] = table[ids[t], col0 : col0 + cols] * scale; out: rows of any stride, f32 or bf16 (default: a new f32 tensor)"""
+    T = ids.shape[0]
+    K = table.shape[1] - col0 if cols is None else cols
+    y = out if out is not None else torch.empty(T, K, dtype=torch.float32, device=table.device)
+    assert y.shape == (T, K) and table.is_contiguous()
+    check(lib().dihip_embed_rows(stream(), ptr(y), dt(y), _rows(y), ptr(ids), ptr(table), dt(table), table.shape[1], int(col0), float(scale),
+                                 T, K), "dihip_embed_rows")
+    return y
+
+
+def rmsnorm(x, gamma, eps, row_idx=None, out=None, gamma_add=0.0, out_scale=1.0):
+    """y = x / rms(x) * (gamma_add + gamma) * out_scale"""
     M = x.shape[0] if row_idx is None else row_idx.shape[0]
     K = gamma.shape[0]
     assert x.shape[1] == K and x.dtype == torch.float32
     y = out if out is not None else torch.empty(M, K, dtype=torch.float32, device=x.device)
-    check(lib().dihip_rmsnorm_strided(stream(), ptr(y), dt(y), _rows(y), ptr(x), _rows(x), ptr(row_idx), ptr(gamma), dt(gamma), float(eps),
-                                      M, K), "dihip_rmsnorm_strided")
+    check(lib().dihip_rmsnorm_strided(stream(), ptr(y), dt(y), _rows(y), ptr(x), _rows(x), ptr(row_idx), ptr(gamma), dt(gamma), float(gamma_add),
+                                      float(out_scale), float(eps), M, K), "dihip_rmsnorm_strided")
     return y
+
+
+def residual_norm_step(x_in, eps, m=None, gamma_m=None, add_m=0.0, x_out=None, gamma_h=None, add_h=0.0, h=None, copy=None):
+    """x_out = x_in + m / rms(m) * (add_m + gamma_m) (m None: x_in itself); copy <- x_out (rows of any stride, f32 or bf16);
+    h <- x_out / rms(x_out) * (add_h + gamma_h) (f32 or bf16).  -> x_out"""
+    T, K = x_in.shape
+    assert x_in.is_contiguous() and x_in.dtype == torch.float32
+    if m is not None:
+        x_out = x_in if x_out is None else x_out
+        assert x_out.is_contiguous() and x_out.shape == (T, K) and m.shape == (T, K) and m.dtype == torch.float32 and gamma_m.shape[0] == K
+    assert h is None or (h.shape == (T, K) and gamma_h.shape[0] == K)
+    assert copy is None or copy.shape == (T, K)
+    g = gamma_m if gamma_m is not None else gamma_h
+    assert gamma_m is None or gamma_h is None or gamma_m.dtype == gamma_h.dtype
+    check(lib().dihip_residual_norm_step(stream(), ptr(x_out), ptr(x_in), ptr(m), _rows(m) if m is not None else 0, ptr(gamma_m), float(add_m),
+                                         ptr(gamma_h), float(add_h), dt(g) if g is not None else F32_CODE, float(eps), ptr(copy),
+                                         dt(copy) if copy is not None else F32_CODE, _rows(copy) if copy is not None else 0, ptr(h),
+                                         dt(h) if h is not None else F32_CODE, _rows(h) if h is not None else 0, T, K), "dihip_residual_norm_step")
+    return x_out if m is not None else x_in
 
 
 def norm_span_append(table, x, gamma, eps, tok_slot, tok_pos):
@@ -166,7 +197,7 @@ def linear_segmented(x, w, seg, row_map, seg_max_rows, R, bias=None, out=None, a
     """rows grouped by owner: w [groups, N, K]; output row r (seg[g] <= r < seg[g + 1]) = x[row_map[r]] . w[g]^T (+ bias[g]);
     seg_max_rows: a host-known bound on one group's rows -> [R, N] f32"""
     groups, N, K = w.shape
-    assert x.shape[1] == K and w.is_contiguous() and seg.dtype == torch.int32 and seg.shape[0] == groups + 1
+    assert x.shape[1] == K and w.is_contiguous() and seg.dtype == torch.int32 and seg.shape[0] >= groups + 1
     y = out if out is not None else torch.empty(R, N, dtype=torch.float32, device=x.device)
     assert y.shape == (R, N)
     check(lib().dihip_linear_segmented(stream(), ptr(x), dt(x), _rows(x), ptr(w), dt(w), ptr(bias), ptr(y), dt(y), _rows(y), R, N, K, groups,
@@ -194,13 +225,14 @@ def add_dyt(x_in, a=None, b=None, norm=None, x_out=None, row_idx=None, want16=Fa
 
 
 def qkv_prep_append(a, q_off, k_off, v_off, H, G, D, DV, qnorm, knorm, eps, freq, rot_dims, layout, mag, lam, vfirst_in, vfirst_out,
-                    ktable, vtable, tok_slot, tok_pos):
-    """norm + rotation of the q / k columns of the rows a (q in place), value mixing, append of k and v to their pages"""
+                    ktable, vtable, tok_slot, tok_pos, maps=1):
+    """norm + rotation of the q / k columns of the rows a (q in place), value mixing, append of k and v to their pages; maps: query
+    vectors per head and key vectors per key head"""
     T = a.shape[0]
-    assert a.dtype == torch.float32 and ktable.row_elems == G * D and vtable.row_elems == G * DV and ktable.dtype == vtable.dtype
+    assert a.dtype == torch.float32 and ktable.row_elems == G * maps * D and vtable.row_elems == G * DV and ktable.dtype == vtable.dtype
     vf = vfirst_in if vfirst_in is not None else vfirst_out
     wn = qnorm if qnorm is not None else knorm
-    check(lib().dihip_qkv_prep_append(stream(), ptr(a), _rows(a), q_off, k_off, v_off, H, G, D, DV, ptr(qnorm), ptr(knorm),
+    check(lib().dihip_qkv_prep_append(stream(), ptr(a), _rows(a), q_off, k_off, v_off, H, G, D, DV, int(maps), ptr(qnorm), ptr(knorm),
                                       dt(wn) if wn is not None else F32_CODE, float(eps), ptr(freq), int(rot_dims), int(layout), float(mag),
                                       float(lam), ptr(vfirst_in), ptr(vfirst_out), _rows(vf) if vf is not None else 0, ptr(ktable.ptrs),
                                       ptr(vtable.ptrs), ktable.max_spans, ktable.span_len, _DT[ktable.dtype], ptr(tok_slot), ptr(tok_pos), T),
@@ -210,38 +242,52 @@ def qkv_prep_append(a, q_off, k_off, v_off, H, G, D, DV, qnorm, knorm, eps, freq
 SINK_NONE, SINK_PER_HEAD, SINK_ZERO = 0, 1, 2
 
 
-def gqa_attn(q, ktable, vtable, tok_slot, tok_pos, H, G, D, DV, scale, sink=None, sink_mode=SINK_NONE, softcap=0.0, gate=None, out=None):
-    """q: f32 [T, >= H * D] rows (a column slice is fine); gate: f32 [T, >= H] or None -> f32 [T, H * DV]"""
+def gqa_attn(q, ktable, vtable, tok_slot, tok_pos, H, G, D, DV, scale, sink=None, sink_mode=SINK_NONE, softcap=0.0, gate=None, out=None,
+             maps=1, window=0, keep_first=0):
+    """q: f32 [T, >= H * maps * D] rows (a column slice is fine); gate: f32 [T, >= H] or None -> f32 [T, H * maps * DV].  window > 0:
+    a row reads the keys less than `window` positions back and the first keep_first keys of its sequence"""
     T = q.shape[0]
-    o = out if out is not None else torch.empty(T, H * DV, dtype=torch.float32, device=q.device)
+    o = out if out is not None else torch.empty(T, H * maps * DV, dtype=torch.float32, device=q.device)
     check(lib().dihip_gqa_attn(stream(), ptr(o), _rows(o), ptr(q), _rows(q), ptr(ktable.ptrs), ptr(vtable.ptrs), ktable.max_spans, ktable.span_len,
                                _DT[ktable.dtype], ptr(sink), dt(sink) if sink is not None else F32_CODE, int(sink_mode), float(softcap or 0.0),
-                               ptr(gate), _rows(gate) if gate is not None else 0, ptr(tok_slot), ptr(tok_pos), T, H, G, D, DV, float(scale)),
-          "dihip_gqa_attn")
+                               ptr(gate), _rows(gate) if gate is not None else 0, ptr(tok_slot), ptr(tok_pos), T, H, G, D, DV, float(scale),
+                               int(maps), int(window or 0), int(keep_first or 0)), "dihip_gqa_attn")
     return o
 
 
-def gqa_attn_mc_supported(ktable, vtable, G):
-    return bool(lib().dihip_gqa_attn_mc_supported(ktable.row_elems // G, vtable.row_elems // G, ktable.span_len, _DT[ktable.dtype]))
+def gqa_attn_mc_supported(D, DV, table):
+    """head sizes D / DV on pages like those of `table`"""
+    return bool(lib().dihip_gqa_attn_mc_supported(int(D), int(DV), table.span_len, _DT[table.dtype]))
 
 
 def gqa_attn_mc(q, ktable, vtable, tok_pos, ent_slot, ent_row0, ent_count, max_count, max_pos, H, G, D, DV, scale, sink=None,
-                sink_mode=SINK_NONE, softcap=0.0, gate=None, out=None, nsplit=None):
+                sink_mode=SINK_NONE, softcap=0.0, gate=None, out=None, nsplit=None, maps=1, window=0, keep_first=0):
     """the matrix-core form (bf16 pages); max_count / max_pos: the largest portion and position of the step (host numbers)"""
     T, E = q.shape[0], ent_slot.shape[0]
-    o = out if out is not None else torch.empty(T, H * DV, dtype=torch.float32, device=q.device)
+    window, keep_first = int(window or 0), int(keep_first or 0)
+    o = out if out is not None else torch.empty(T, H * maps * DV, dtype=torch.float32, device=q.device)
     if nsplit is None:       # fill the chip: ~2 workgroups per CU; at least 2 key tiles (64 keys) per workgroup
-        blocks = max(1, E * G * ((max_count * (H // G) + 63) // 64))
-        nsplit = max(1, min(512 // blocks, (max_pos + 1 + 63) // 64))
+        blocks = max(1, E * G * maps * ((max_count * (H // G) + 63) // 64))
+        keys = min(max_pos + 1, window + keep_first) if window > 0 else max_pos + 1
+        nsplit = max(1, min(512 // blocks, (keys + 63) // 64))
     ws = None
     if nsplit > 1:
-        ws = torch.empty(int(lib().dihip_gqa_attn_mc_workspace_bytes(T, H, DV, nsplit)), dtype=torch.uint8, device=q.device)
+        ws = torch.empty(int(lib().dihip_gqa_attn_mc_workspace_bytes(T, H * maps, DV, nsplit)), dtype=torch.uint8, device=q.device)
     check(lib().dihip_gqa_attn_mc(stream(), ptr(o), _rows(o), ptr(q), _rows(q), ptr(ktable.ptrs), ptr(vtable.ptrs), ktable.max_spans,
                                   ktable.span_len, ptr(sink), dt(sink) if sink is not None else F32_CODE, int(sink_mode), float(softcap or 0.0),
                                   ptr(gate), _rows(gate) if gate is not None else 0, ptr(tok_pos), ptr(ent_slot), ptr(ent_row0), ptr(ent_count),
-                                  E, int(max_count), T, H, G, D, DV, float(scale), int(nsplit), ptr(ws), ws.numel() if ws is not None else 0),
-          "dihip_gqa_attn_mc")
+                                  E, int(max_count), T, H, G, D, DV, float(scale), int(maps), window, keep_first, int(nsplit), ptr(ws),
+                                  ws.numel() if ws is not None else 0), "dihip_gqa_attn_mc")
     return o
+
+
+def maps_diff_norm(x, lam, out_scale, eps, H, DV, out=None):
+    """x: f32 [T, H * 2 * DV] (two maps per head side by side) -> (first - lam * second) / its root mean square * out_scale, [T, H * DV]"""
+    T = x.shape[0]
+    y = out if out is not None else torch.empty(T, H * DV, dtype=torch.float32, device=x.device)
+    check(lib().dihip_maps_diff_norm(stream(), ptr(y), dt(y), _rows(y), ptr(x), _rows(x), float(lam), float(out_scale), float(eps), T, H, DV),
+          "dihip_maps_diff_norm")
+    return y
 
 
 CHUNKED_GLA_ROWS = 128   # portions from this length on run as chunks side by side
@@ -270,7 +316,11 @@ def head_rmsnorm_mul(x, gamma, eps, H, DV, mul=None, out=None):
     return y
 
 
-def moe_route(logits, top):
+ROUTE_CHOSEN_SOFTMAX, ROUTE_SCORES = 0, 1      # weights = softmax over the chosen logits / the chosen softmax scores over their sum
+UNIT_CLAMPED, UNIT_SILU = 0, 1
+
+
+def moe_route(logits, top, scoring=ROUTE_CHOSEN_SOFTMAX, correction=None):
     """-> ids [T, top] i32, wts [T, top] f32, seg [E + 1], src_row [T * top], dst [T * top]"""
     T, E = logits.shape
     dev = logits.device
@@ -278,21 +328,25 @@ def moe_route(logits, top):
     ids, src_row, dst = ints[: T * top], ints[T * top: 2 * T * top], ints[2 * T * top: 3 * T * top]
     counts, seg = ints[3 * T * top: 3 * T * top + E], ints[3 * T * top + E:]
     wts = torch.empty(T, top, dtype=torch.float32, device=dev)
+    assert correction is None or (correction.shape == (E,) and correction.is_contiguous())
     check(lib().dihip_seq_moe_route(stream(), ptr(logits), _rows(logits), ptr(ids), ptr(wts), ptr(counts), ptr(seg), ptr(src_row), ptr(dst),
-                                    T, E, int(top)), "dihip_seq_moe_route")
+                                    T, E, int(top), int(scoring), ptr(correction), dt(correction) if correction is not None else F32_CODE),
+          "dihip_seq_moe_route")
     return ids.view(T, top), wts, seg, src_row, dst
 
 
-def moe_glu(gu, F, limit, slope, out):
+def moe_glu(gu, F, limit, slope, out, unit=UNIT_CLAMPED):
     R = gu.shape[0]
-    check(lib().dihip_seq_moe_glu(stream(), ptr(out), dt(out), _rows(out), ptr(gu), _rows(gu), R, F, float(limit), float(slope)),
+    check(lib().dihip_seq_moe_glu(stream(), ptr(out), dt(out), _rows(out), ptr(gu), _rows(gu), R, F, float(limit), float(slope), int(unit)),
           "dihip_seq_moe_glu")
     return out
 
 
-def moe_combine(rows, dst, wts, T, top, out=None):
+def moe_combine(rows, dst, wts, T, top, out=None, ids=None, n_real=0, own=None, add=None):
+    """ids / n_real / own: choices >= n_real are identity experts, their row is own[t] (f32 or bf16); add: f32 rows added per token"""
     K = rows.shape[1]
     o = out if out is not None else torch.empty(T, K, dtype=torch.float32, device=rows.device)
-    check(lib().dihip_seq_moe_combine(stream(), ptr(o), _rows(o), ptr(rows), _rows(rows), ptr(dst), ptr(wts), T, int(top), K),
-          "dihip_seq_moe_combine")
+    check(lib().dihip_seq_moe_combine(stream(), ptr(o), _rows(o), ptr(rows), _rows(rows), ptr(dst), ptr(wts), T, int(top), K, ptr(ids), int(n_real),
+                                      ptr(own), dt(own) if own is not None else F32_CODE, _rows(own) if own is not None else 0, ptr(add),
+                                      _rows(add) if add is not None else 0), "dihip_seq_moe_combine")
     return o

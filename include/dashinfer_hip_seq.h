@@ -56,36 +56,42 @@ int dihip_add_dyt(void* stream, float* x_out, const float* x_in, const float* a,
                   const int32_t* row_idx, float alpha, const void* w, const void* bias, int w_dtype, float* h, void* h16,
                   int M, int K);
 
-/* Grouped-query attention, step 1: per token the rows qkv[t] hold q [H, D] at column q_off, k [G, D] at k_off, v [G, DV] at
- * v_off (f32).  Every query and key head is divided by its root mean square and scaled by qnorm / knorm [D] (NULL: no norm),
+/* Grouped-query attention, step 1: per token the rows qkv[t] hold q [H, maps, D] at column q_off, k [G, maps, D] at k_off,
+ * v [G, DV] at v_off (f32; maps = the softmax maps per head, 1 for ordinary attention).  Every query and key head is divided by its root mean square and scaled by qnorm / knorm [D] (NULL: no norm),
  * then rotated on its first rot_dims dimensions by the angles tok_pos[t] * freq[i] (f32 product; layout 0: dimension 2i
  * with 2i + 1, layout 1: i with i + rot_dims / 2; cos and sin times `mag`).  Queries are written back in place, keys go to
- * the key pages (rows of G * D elements of cache_dtype), values to the value pages (rows of G * DV) after
+ * the key pages (rows of G * maps * D elements of cache_dtype), values to the value pages (rows of G * DV) after
  *   v <- (1 - lam) v + lam vfirst_in[t]   (vfirst_in NULL: v as it is);   vfirst_out[t] <- v   (NULL: not kept). */
-int dihip_qkv_prep_append(void* stream, float* qkv, long ld, int q_off, int k_off, int v_off, int H, int G, int D, int DV,
+int dihip_qkv_prep_append(void* stream, float* qkv, long ld, int q_off, int k_off, int v_off, int H, int G, int D, int DV, int maps,
                           const void* qnorm, const void* knorm, int w_dtype, float eps, const float* freq, int rot_dims,
                           int layout, float mag, float lam, const float* vfirst_in, float* vfirst_out, long ldvf,
                           void* const* kspans, void* const* vspans, int span_stride, int span_len, int cache_dtype,
                           const int32_t* tok_slot, const int32_t* tok_pos, int T);
 
 /* step 2: causal attention of every row over its sequence's pages; query head h reads key/value head h / (H / G):
- *   s_j = scale * q[t, h] . k_j,  softcap > 0: s_j <- softcap * tanh(s_j / softcap),  j <= tok_pos[t]
+ *   s_j = scale * q[t, h, m] . k_j[m],  softcap > 0: s_j <- softcap * tanh(s_j / softcap),
+ *   over the keys j <= p = tok_pos[t] with  p - j < window  or  j < keep_first  (window <= 0: every j <= p)
  *   p = softmax over {s_j} and, with sink_mode 1 / 2, one more logit sink[h] / 0 that has no value
- *   out[t, h] = gate[t, h] * sum_j p_j v_j   (gate NULL: 1)
- * q [T, H, D], out [T, H, DV] f32.  Every product and sum in f32. */
+ *   out[t, h, m] = gate[t, h] * sum_j p_j v_j   (gate NULL: 1)
+ * for every map m < maps of the head (each a softmax of its own over the same values).
+ * q [T, H, maps, D], out [T, H, maps, DV] f32.  Every product and sum in f32. */
 int dihip_gqa_attn(void* stream, float* out, long ldo, const float* q, long ldq, void* const* kspans, void* const* vspans,
                    int span_stride, int span_len, int cache_dtype, const void* sink, int w_dtype, int sink_mode, float softcap,
                    const float* gate, long ldg, const int32_t* tok_slot, const int32_t* tok_pos, int T, int H, int G, int D,
-                   int DV, float scale);
+                   int DV, float scale, int maps, int window, int keep_first);
 /* the same on the matrix cores for bf16 pages (D, DV multiples of 8 up to 256 / 128, span_len a multiple of 32): rows given
  * as portions, the key walk split over nsplit workgroups (see dihip_latent_window_attn_mc) */
 int dihip_gqa_attn_mc_supported(int D, int DV, int span_len, int cache_dtype);
-size_t dihip_gqa_attn_mc_workspace_bytes(int T, int H, int DV, int nsplit);
+size_t dihip_gqa_attn_mc_workspace_bytes(int T, int H_times_maps, int DV, int nsplit);
 int dihip_gqa_attn_mc(void* stream, float* out, long ldo, const float* q, long ldq, void* const* kspans, void* const* vspans,
                       int span_stride, int span_len, const void* sink, int w_dtype, int sink_mode, float softcap,
                       const float* gate, long ldg, const int32_t* tok_pos, const int32_t* ent_slot, const int32_t* ent_row0,
                       const int32_t* ent_count, int E, int max_count, int T, int H, int G, int D, int DV, float scale,
-                      int nsplit, void* ws, size_t ws_bytes);
+                      int maps, int window, int keep_first, int nsplit, void* ws, size_t ws_bytes);
+/* two maps per head -> one (differential attention):  d = x[t, h, 0] - lam * x[t, h, 1];
+ *   y[t, h, :] = d / sqrt(mean(d^2) + eps) * out_scale        x f32 [T, H, 2, DV], y [T, H, DV] of y_dtype */
+int dihip_maps_diff_norm(void* stream, void* y, int y_dtype, long ldy, const float* x, long ldx, float lam, float out_scale,
+                         float eps, int T, int H, int DV);
 
 /* Gated linear attention, per head and portion, rows in order, f32:
  *   alpha = sigmoid(z[t, h, :])^(1 / tau);   S <- diag(alpha) S + k[t, h] v[t, h]^T;   out[t, h] = S^T (q[t, h] * q_scale)
@@ -102,24 +108,43 @@ int dihip_head_rmsnorm_mul(void* stream, void* y, int y_dtype, long ldy, const f
                            int w_dtype, float eps, const float* mul, long ldm, int T, int H, int DV);
 
 /* Mixture of experts: per token the `top` experts of largest logit (ties: the lower index) and the softmax over the chosen
- * logits -> ids / wts [T, top]; the T * top (token, choice) pairs grouped by expert -> seg [E + 1], src_row [T * top] (the
+ * logits (scoring 0), or scores = softmax over all E logits, the `top` experts of largest score + correction[e] (correction
+ * [E] of w_dtype, NULL: none) and weights = their scores / (the sum of their scores + 1e-20) (scoring 1) -> ids / wts [T, top]; the T * top (token, choice) pairs grouped by expert -> seg [E + 1], src_row [T * top] (the
  * token a sorted row reads), dst [T * top] (the sorted row of pair t * top + k); counts: [E] scratch. */
 int dihip_seq_moe_route(void* stream, const float* logits, long ldl, int32_t* ids, float* wts, int32_t* counts, int32_t* seg,
-                    int32_t* src_row, int32_t* dst, int T, int E, int top);
-/* y[r, c] = g * sigmoid(slope * g) * (u + 1),  g = min(gu[r, c], limit),  u = clamp(gu[r, F + c], -limit, limit) */
+                    int32_t* src_row, int32_t* dst, int T, int E, int top, int scoring, const void* correction, int w_dtype);
+/* unit 0: y[r, c] = g * sigmoid(slope * g) * (u + 1),  g = min(gu[r, c], limit),  u = clamp(gu[r, F + c], -limit, limit)
+ * unit 1: y[r, c] = silu(gu[r, c]) * gu[r, F + c] */
 int dihip_seq_moe_glu(void* stream, void* y, int y_dtype, long ldy, const float* gu, long ldgu, int R, int F, float limit,
-                  float slope);
-/* out[t] = sum_k wts[t, k] * rows[dst[t * top + k]],  k ascending */
+                  float slope, int unit);
+/* out[t] = sum_k wts[t, k] * rows[dst[t * top + k]] (+ add[t]),  k ascending.  ids != NULL: a choice ids[t * top + k] >= n_real
+ * is an identity expert, its row is the token's own row own[t] (of own_dtype).  add NULL: nothing added. */
 int dihip_seq_moe_combine(void* stream, float* out, long ldo, const float* rows, long ldr, const int32_t* dst, const float* wts,
-                      int T, int top, int K);
+                      int T, int top, int K, const int32_t* ids, int n_real, const void* own, int own_dtype, long ldown,
+                      const float* add, long ldadd);
 
 /* h[t, :] = float(table[ids[t], :]) + float(table2[rows2[t], :])   (table2 NULL: the first term alone) */
 int dihip_embed_sum(void* stream, float* h, const int32_t* ids, const void* table, const int32_t* rows2,
                     const void* table2, int w_dtype, int T, int K);
 
-/* y[i, :] = x[r, :] / sqrt(mean(x[r, :]^2) + eps) * gamma,  r = row_idx ? row_idx[i] : i;  x f32 rows of stride ldx */
+/* y[t, :] = float(table[ids[t], col0 .. col0 + K)) * scale;  table rows of ldt elements of w_dtype, y rows of ldy of y_dtype */
+int dihip_embed_rows(void* stream, void* y, int y_dtype, long ldy, const int32_t* ids, const void* table, int w_dtype,
+                     long ldt, long col0, float scale, int T, int K);
+
+/* y[i, :] = x[r, :] / sqrt(mean(x[r, :]^2) + eps) * (gamma_add + gamma) * out_scale,  r = row_idx ? row_idx[i] : i;  x f32 rows
+ * of stride ldx  (gamma_add 1: a weight stored as its deviation from one) */
 int dihip_rmsnorm_strided(void* stream, void* y, int y_dtype, long ldy, const float* x, long ldx,
-                          const int32_t* row_idx, const void* gamma, int w_dtype, float eps, int M, int K);
+                          const int32_t* row_idx, const void* gamma, int w_dtype, float gamma_add, float out_scale, float eps,
+                          int M, int K);
+
+/* The residual step of a layer with a norm before and after every sublayer, fused with the next sublayer's input norm:
+ *   xo = x_in + m / rms(m) * (add_m + gamma_m)      (m NULL: xo = x_in, x_out unused)
+ *   x_out = xo;   xc = xo  (a copy of xc_dtype in rows of stride ldc; NULL: none);
+ *   h = xo / rms(xo) * (add_h + gamma_h)            (of h_dtype, rows of stride ldh; NULL: none)
+ * rms(v) = sqrt(mean(v^2) + eps).  x_in / x_out: contiguous [T, K] f32 (may alias). */
+int dihip_residual_norm_step(void* stream, float* x_out, const float* x_in, const float* m, long ldm, const void* gamma_m,
+                             float add_m, const void* gamma_h, float add_h, int w_dtype, float eps, void* xc, int xc_dtype,
+                             long ldc, void* h, int h_dtype, long ldh, int T, int K);
 /* the same norm, written into the paged cache at (tok_slot[t], tok_pos[t]): span row of K elements of cache_dtype */
 int dihip_norm_span_append(void* stream, void* const* spans, int span_stride, int span_len, int cache_dtype,
                            const float* x, long ldx, const void* gamma, int w_dtype, float eps,
