@@ -195,6 +195,65 @@ __global__ __launch_bounds__(256) void add_dyt_kernel(float* x_out, const float*
   }
 }
 
+// The same step for rows of up to 1024 * VPT elements (a multiple of 4, 16-byte aligned rows): the row stays in registers, every
+// operand is read once and all of a thread's loads are in flight together -- two memory round trips and two block sums per row.
+template <int WT, int VPT>
+__global__ __launch_bounds__(256) void residual_norm_step_reg_kernel(float* x_out, const float* x_in, const float* __restrict__ m, long ldm,
+                                                                     const void* __restrict__ gamma_m, float add_m,
+                                                                     const void* __restrict__ gamma_h, float add_h, float eps,
+                                                                     void* __restrict__ xc, int cdt, long ldc, void* __restrict__ h, int hdt,
+                                                                     long ldh, int K) {
+  __shared__ float red[4];
+  const int t = blockIdx.x;
+  const size_t row = (size_t)t * K;
+  const f32x4_t z4 = {0.f, 0.f, 0.f, 0.f};
+  f32x4_t xv[VPT], mv[VPT];
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    const int k = (threadIdx.x + 256 * i) * 4;
+    xv[i] = k < K ? *reinterpret_cast<const f32x4_t*>(x_in + row + k) : z4;
+    mv[i] = m && k < K ? *reinterpret_cast<const f32x4_t*>(m + (size_t)t * ldm + k) : z4;
+  }
+  if (m) {
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < VPT; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) ss = __builtin_fmaf(mv[i][j], mv[i][j], ss);
+    const float inv_m = 1.f / sqrtf(block256_sum(ss, red) / (float)K + eps);
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+      const int k = (threadIdx.x + 256 * i) * 4;
+      if (k < K) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) xv[i][j] += mv[i][j] * inv_m * (add_m + load_ft<WT>(gamma_m, k + j));
+        *reinterpret_cast<f32x4_t*>(x_out + row + k) = xv[i];
+      }
+    }
+  }
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    const int k = (threadIdx.x + 256 * i) * 4;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) ss = __builtin_fmaf(xv[i][j], xv[i][j], ss);
+    if (xc && k < K) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) st_any(xc, (size_t)t * ldc + k + j, cdt, xv[i][j]);
+    }
+  }
+  if (!h) return;
+  const float inv = 1.f / sqrtf(block256_sum(ss, red) / (float)K + eps);
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    const int k = (threadIdx.x + 256 * i) * 4;
+    if (k < K) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) st_any(h, (size_t)t * ldh + k + j, hdt, xv[i][j] * inv * (add_h + load_ft<WT>(gamma_h, k + j)));
+    }
+  }
+}
+
 // ------------------------------------------------------------------------------------------------ latent attention
 // One workgroup per row, its 4 waves take the heads in turn.  A wave walks the row's window in chunks of 64 keys: lane j
 // scores key j (f32 dot over the R latent elements, r ascending), the chunk joins the running softmax (which starts at
@@ -465,6 +524,23 @@ int dihip_residual_norm_step(void* stream, float* x_out, const float* x_in, cons
                     seq_dtype_ok(w_dtype) && seq_dtype_ok(xc_dtype) && seq_dtype_ok(h_dtype), DIHIP_PARAM_ERROR, "residual_norm_step: bad argument");
   if (T == 0) return DIHIP_SUCCESS;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  const auto al16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
+  if (K % 4 == 0 && K <= 8192 && al16(x_in) && (!m || (al16(m) && ldm % 4 == 0 && al16(x_out)))) {   // the row fits the registers
+    auto go = [&](auto wt, auto vpt) {
+      constexpr int WT = decltype(wt)::value, VPT = decltype(vpt)::value;
+      hipLaunchKernelGGL((residual_norm_step_reg_kernel<WT, VPT>), dim3(T), dim3(256), 0, s, x_out, x_in, m, ldm, gamma_m, add_m, gamma_h, add_h, eps,
+                         xc, xc_dtype, ldc, h, h_dtype, ldh, K);
+    };
+    auto by_k = [&](auto wt) {
+      if (K <= 1024) go(wt, std::integral_constant<int, 1>{});
+      else if (K <= 2048) go(wt, std::integral_constant<int, 2>{});
+      else if (K <= 4096) go(wt, std::integral_constant<int, 4>{});
+      else go(wt, std::integral_constant<int, 8>{});
+    };
+    if (w_dtype == DIHIP_F32) by_k(std::integral_constant<int, DIHIP_F32>{});
+    else by_k(std::integral_constant<int, DIHIP_BF16>{});
+    return launch_status();
+  }
   if (w_dtype == DIHIP_F32) hipLaunchKernelGGL(residual_norm_step_kernel<DIHIP_F32>, dim3(T), dim3(256), 0, s, x_out, x_in, m, ldm, gamma_m, add_m, gamma_h, add_h, eps, xc, xc_dtype, ldc, h, h_dtype, ldh, K);
   else hipLaunchKernelGGL(residual_norm_step_kernel<DIHIP_BF16>, dim3(T), dim3(256), 0, s, x_out, x_in, m, ldm, gamma_m, add_m, gamma_h, add_h, eps, xc, xc_dtype, ldc, h, h_dtype, ldh, K);
   return launch_status();

@@ -140,6 +140,7 @@ class Tobilorn:
         if self.loop:     # [x | x0] as the pass entry reads it; x0 is written once
             cat = torch.empty(T, 2 * W, dtype=act, device=dev)
             so.embed_rows(ctx.ids, self.embed, scale=self.embed_scale, out=cat[:, W:])
+        side = so.embed_rows(ctx.ids, self.side_embed) if self.side_dim else None      # every layer's part of the tokens' side rows, once
         pending = None    # (m, gamma, gamma_add) of the sublayer that ran last
 
         def advance(norm=None, raw=False, left=False):
@@ -164,8 +165,8 @@ class Tobilorn:
                 pending = (L.ff(ctx, advance(norm=L.norm2)), L.norm2b, 1.0)
             if L.side is not None:
                 S = L.side
-                e = so.embed_rows(ctx.ids, self.side_embed, col0=S.col0, cols=S.dim)
-                g = so.linear(advance(raw=True), S.gate, act="gelu_tanh", mul=e, math=ctx.math, out=ctx.act_buffer(S.dim))
+                g = so.linear(advance(raw=True), S.gate, act="gelu_tanh", mul=side[:, S.col0: S.col0 + S.dim], math=ctx.math,
+                              out=ctx.act_buffer(S.dim))
                 pending = (so.linear(g, S.proj, math=ctx.math), S.norm, 0.0)
             if ctx.taps is not None:
                 advance()

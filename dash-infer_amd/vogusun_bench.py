@@ -19,9 +19,9 @@ SIZES = {
 PATTERN = ("attention+dense", "gla+moe", "attention_2+dense", "attention+moe", "gla+dense", "attention_2+moe")
 
 
-def random_model(size, device="cuda", seed=0):
-    """config + bf16 tensors on the device (torch generator: nothing of it is trained or loaded)"""
-    s = SIZES[size]
+def random_model(size, device="cuda", seed=0, pattern=PATTERN):
+    """config + bf16 tensors on the device (torch generator: nothing of it is trained or loaded); pattern: the layers' kinds"""
+    s = SIZES[size] if isinstance(size, str) else size
     g = torch.Generator(device=device).manual_seed(seed)
     W = s["width"]
 
@@ -38,7 +38,7 @@ def random_model(size, device="cuda", seed=0):
     t = {"embed": r(s["vocab"], W, sd=1.0), "head": r(s["vocab"], W)}
     norm("final.norm")
     H, G, D, V = s["heads"], s["kv_heads"], s["dim"], s["vdim"]
-    for i, spec in enumerate(PATTERN):
+    for i, spec in enumerate(pattern):
         kind, _, ff = spec.partition("+")
         p = f"l{i}."
         norm(p + "norm1")

@@ -44,7 +44,7 @@ def test_offset_norm_with_rows_and_scale(so):
     assert rel_err(plain.cpu().numpy(), ot.unit_rms(x, 1e-4) * w) < 2e-6
 
 
-@pytest.mark.parametrize("K", [72, 1024 + 41])
+@pytest.mark.parametrize("K", [72, 1024 + 41, 5000])     # a row in registers, the generic kernel (no multiple of 4), the widest register form
 def test_residual_step_fused_with_the_next_norm(so, K):
     rng = np.random.default_rng(1)
     T, eps = 19, 1e-5
