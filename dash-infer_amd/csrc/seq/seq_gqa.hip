@@ -414,14 +414,9 @@ __global__ __launch_bounds__(256) void gqa_attn_mc_kernel(GqaArgs a) {
   }
 }
 
-// one workgroup per (row, head): the splits' (maximum, denominator, sums) records -> the row's output
-__global__ __launch_bounds__(256) void gqa_attn_merge_kernel(float* __restrict__ out, long ldo, const float* __restrict__ ws, int nsplit,
-                                                             int rows_total, int H, int maps, int DV, int Vp, const float* __restrict__ gate, long ldg) {
-  __shared__ float wgt[1024];
-  __shared__ float red[4];
-  const int gi = blockIdx.x, HQ = H * maps, t = gi / HQ, hq = gi - t * HQ, h = hq / maps;
-  const size_t rec = (size_t)Vp + 4, stride = (size_t)rows_total * rec;
-  const float* base = ws + (size_t)gi * rec;
+// The splits' (maximum, denominator, sums) records of one (row, query vector) -> column threadIdx.x of its softmax-weighted sum
+// (0 for threads past DV; DV <= 256).  wgt / red: LDS scratch of the workgroup; the call synchronises it.
+__device__ __forceinline__ float merge_splits(const float* __restrict__ base, size_t stride, int nsplit, int Vp, int DV, float* wgt, float* red) {
   float mloc[4], lloc[4], mx = -INFINITY;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
@@ -431,6 +426,7 @@ __global__ __launch_bounds__(256) void gqa_attn_merge_kernel(float* __restrict__
     mx = fmaxf(mx, mloc[i]);
   }
   mx = wave_max(mx);
+  __syncthreads();                   // wgt / red of an earlier call are no longer read
   if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = mx;
   __syncthreads();
   mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
@@ -443,13 +439,40 @@ __global__ __launch_bounds__(256) void gqa_attn_merge_kernel(float* __restrict__
     den = __builtin_fmaf(w, lloc[i], den);
   }
   den = block256_sum(den, red);      // (its barriers publish wgt)
-  const float inv = (gate ? gate[(size_t)t * ldg + h] : 1.f) / den;
-  for (int r = threadIdx.x; r < DV; r += 256) {
-    float acc = 0.f;
+  float acc = 0.f;
+  const int r = threadIdx.x;
+  if (r < DV) {
 #pragma unroll 8
     for (int s = 0; s < nsplit; ++s) acc = __builtin_fmaf(wgt[s], base[s * stride + r], acc);
-    out[(size_t)t * ldo + (size_t)hq * DV + r] = acc * inv;
   }
+  return acc / den;
+}
+
+// one workgroup per (row, query vector)
+__global__ __launch_bounds__(256) void gqa_attn_merge_kernel(float* __restrict__ out, long ldo, const float* __restrict__ ws, int nsplit,
+                                                             int rows_total, int H, int maps, int DV, int Vp, const float* __restrict__ gate, long ldg) {
+  __shared__ float wgt[1024];
+  __shared__ float red[4];
+  const int gi = blockIdx.x, HQ = H * maps, t = gi / HQ, hq = gi - t * HQ, h = hq / maps;
+  const size_t rec = (size_t)Vp + 4;
+  const float v = merge_splits(ws + (size_t)gi * rec, (size_t)rows_total * rec, nsplit, Vp, DV, wgt, red);
+  if (threadIdx.x < DV) out[(size_t)t * ldo + (size_t)hq * DV + threadIdx.x] = v * (gate ? gate[(size_t)t * ldg + h] : 1.f);
+}
+
+// one workgroup per (row, head) of two maps: both merged, then d = first - lam * second, y = d / sqrt(mean(d^2) + eps) * out_scale
+__global__ __launch_bounds__(256) void gqa_attn_merge_diff_kernel(void* __restrict__ y, int ydt, long ldy, const float* __restrict__ ws, int nsplit,
+                                                                  int rows_total, int H, int DV, int Vp, const float* __restrict__ gate, long ldg,
+                                                                  float lam, float out_scale, float eps) {
+  __shared__ float wgt[1024];
+  __shared__ float red[4];
+  const int gi = blockIdx.x, t = gi / H, h = gi - t * H;
+  const size_t rec = (size_t)Vp + 4, stride = (size_t)rows_total * rec;
+  const float* base = ws + ((size_t)t * H * 2 + (size_t)h * 2) * rec;
+  const float a1 = merge_splits(base, stride, nsplit, Vp, DV, wgt, red);
+  const float a2 = merge_splits(base + rec, stride, nsplit, Vp, DV, wgt, red);
+  const float d = (a1 - lam * a2) * (gate ? gate[(size_t)t * ldg + h] : 1.f);
+  const float inv = out_scale / sqrtf(block256_sum(d * d, red) / (float)DV + eps);
+  if (threadIdx.x < DV) st_any(y, (size_t)t * ldy + (size_t)h * DV + threadIdx.x, ydt, d * inv);
 }
 
 }  // namespace
@@ -533,7 +556,7 @@ int dihip_gqa_attn_mc(void* stream, float* out, long ldo, const float* q, long l
                       int span_stride, int span_len, const void* sink, int w_dtype, int sink_mode, float softcap, const float* gate,
                       long ldg, const int32_t* tok_pos, const int32_t* ent_slot, const int32_t* ent_row0, const int32_t* ent_count, int E,
                       int max_count, int T, int H, int G, int D, int DV, float scale, int maps, int window, int keep_first, int nsplit,
-                      void* ws, size_t ws_bytes) {
+                      void* ws, size_t ws_bytes, void* diff_out, int diff_dtype, long ldd, float lam, float out_scale, float eps) {
   if (int rc = gqa_check("gqa_attn_mc", out, ldo, q, ldq, kspans, vspans, span_stride, span_len, sink, w_dtype, sink_mode, gate, ldg, H, G, D, DV, maps, keep_first)) return rc;
   DIHIP_REQUIRE(dihip_gqa_attn_mc_supported(D, DV, span_len, DIHIP_BF16), DIHIP_PARAM_ERROR,
                 "gqa_attn_mc: head sizes %d / %d (multiples of 8 up to 256 / 128) or span_len %d (a multiple of 32) not served", D, DV, span_len);
@@ -542,6 +565,8 @@ int dihip_gqa_attn_mc(void* stream, float* out, long ldo, const float* q, long l
   DIHIP_REQUIRE((reinterpret_cast<uintptr_t>(out) & 15u) == 0 && (reinterpret_cast<uintptr_t>(q) & 15u) == 0, DIHIP_PARAM_ERROR,
                 "gqa_attn_mc: q / out must be 16-byte aligned");
   DIHIP_REQUIRE(nsplit >= 1 && nsplit <= 1024 && (long)E * G * maps <= 65535, DIHIP_PARAM_ERROR, "gqa_attn_mc: bad split / portion count");
+  DIHIP_REQUIRE(!diff_out || (maps == 2 && ldd >= (long)H * DV && seq_dtype_ok(diff_dtype)), DIHIP_PARAM_ERROR,
+                "gqa_attn_mc: the difference of the maps needs two maps and rows of H * DV elements");
   DIHIP_REQUIRE(ws_bytes >= dihip_gqa_attn_mc_workspace_bytes(T, H * maps, DV, nsplit) && (nsplit == 1 || ws), DIHIP_PARAM_ERROR,
                 "gqa_attn_mc: workspace too small");
   if (E == 0 || max_count == 0) return DIHIP_SUCCESS;
@@ -562,7 +587,14 @@ int dihip_gqa_attn_mc(void* stream, float* out, long ldo, const float* q, long l
   if (D <= 64) by_v(std::integral_constant<int, 64>{});
   else if (D <= 128) by_v(std::integral_constant<int, 128>{});
   else by_v(std::integral_constant<int, 256>{});
-  if (nsplit > 1) hipLaunchKernelGGL(gqa_attn_merge_kernel, dim3(T * H * maps), dim3(256), 0, s, out, ldo, (const float*)ws, nsplit, T * H * maps, H, maps, DV, Vp, gate, ldg);
+  if (nsplit > 1 && diff_out)      // the merge of both maps, their difference and its norm in one launch
+    hipLaunchKernelGGL(gqa_attn_merge_diff_kernel, dim3(T * H), dim3(256), 0, s, diff_out, diff_dtype, ldd, (const float*)ws, nsplit, T * H * maps, H, DV,
+                       Vp, gate, ldg, lam, out_scale, eps);
+  else if (nsplit > 1)
+    hipLaunchKernelGGL(gqa_attn_merge_kernel, dim3(T * H * maps), dim3(256), 0, s, out, ldo, (const float*)ws, nsplit, T * H * maps, H, maps, DV, Vp, gate, ldg);
+  else if (diff_out)
+    hipLaunchKernelGGL(maps_diff_norm_kernel, dim3((unsigned)(((long)T * H + 3) / 4)), dim3(256), 0, s, diff_out, diff_dtype, ldd, out, ldo, lam, out_scale,
+                       eps, T * H, H, DV);
   return launch_status();
 }
 

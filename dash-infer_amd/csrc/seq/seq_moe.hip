@@ -12,17 +12,18 @@
 namespace dihip {
 namespace {
 
-// scoring 1: every logit is read three times (maximum, denominator, choice): E is small and the row stays in cache
-__global__ __launch_bounds__(256) void moe_route_scores_kernel(const float* __restrict__ logits, long ldl, const void* __restrict__ corr, int cdt,
-                                                               int32_t* __restrict__ ids, float* __restrict__ wts, int T, int E, int top) {
-  const int t = blockIdx.x * 256 + threadIdx.x;
-  if (t >= T) return;
-  const float* z = logits + (size_t)t * ldl;
-  float zmax = -INFINITY, den = 0.f;
-  for (int e = 0; e < E; ++e) zmax = fmaxf(zmax, z[e]);
-  for (int e = 0; e < E; ++e) den += expf(z[e] - zmax);
-  float best[32];
-  int bi[32];
+// One token's choice.  scoring 0: the `top` largest logits (ties: the lower index), weights = softmax over them alone.  scoring 1:
+// scores = softmax over all E logits, the choice by score + correction, weights = the chosen scores over their sum.  (Every logit
+// is read a few times: E is small and the row stays in cache.)
+template <int SCORING>
+__device__ __forceinline__ void route_token(const float* __restrict__ z, const void* __restrict__ corr, int cdt, int E, int top, int (&bi)[32],
+                                            float (&w)[32]) {
+  float zmax = -INFINITY, den = 1.f;
+  if (SCORING == 1) {
+    for (int e = 0; e < E; ++e) zmax = fmaxf(zmax, z[e]);
+    den = 0.f;
+    for (int e = 0; e < E; ++e) den += expf(z[e] - zmax);
+  }
   float sum = 0.f;
   for (int k = 0; k < top; ++k) {
     float bv = -INFINITY, bs = 0.f;
@@ -30,43 +31,78 @@ __global__ __launch_bounds__(256) void moe_route_scores_kernel(const float* __re
     for (int e = 0; e < E; ++e) {
       bool used = false;
       for (int j = 0; j < k; ++j) used |= bi[j] == e;
-      const float sc = expf(z[e] - zmax) / den;
-      const float v = sc + (corr ? ld_any(corr, e, cdt) : 0.f);
+      float v = z[e], sc = v;
+      if (SCORING == 1) {
+        sc = expf(v - zmax) / den;
+        v = sc + (corr ? ld_any(corr, e, cdt) : 0.f);
+      }
       if (!used && (bx < 0 || v > bv)) { bv = v; bx = e; bs = sc; }
     }
-    best[k] = bs; bi[k] = bx;
+    w[k] = bs; bi[k] = bx;
     sum += bs;
   }
-  for (int k = 0; k < top; ++k) {
-    ids[(size_t)t * top + k] = bi[k];
-    wts[(size_t)t * top + k] = best[k] / (sum + 1e-20f);
+  if (SCORING == 1) {
+    for (int k = 0; k < top; ++k) w[k] = w[k] / (sum + 1e-20f);
+  } else {
+    float d = 0.f;
+    const float m0 = w[0];
+    for (int k = 0; k < top; ++k) { w[k] = expf(w[k] - m0); d += w[k]; }
+    for (int k = 0; k < top; ++k) w[k] = w[k] / d;
   }
 }
 
-__global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits, long ldl, int32_t* __restrict__ ids,
-                                                        float* __restrict__ wts, int T, int E, int top) {
+template <int SCORING>
+__global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits, long ldl, const void* __restrict__ corr, int cdt,
+                                                        int32_t* __restrict__ ids, float* __restrict__ wts, int T, int E, int top) {
   const int t = blockIdx.x * 256 + threadIdx.x;
   if (t >= T) return;
-  const float* z = logits + (size_t)t * ldl;
-  float best[32];
   int bi[32];
-  for (int k = 0; k < top; ++k) {
-    float bv = -INFINITY;
-    int bx = -1;
-    for (int e = 0; e < E; ++e) {
-      bool used = false;
-      for (int j = 0; j < k; ++j) used |= bi[j] == e;
-      const float v = z[e];
-      if (!used && (bx < 0 || v > bv)) { bv = v; bx = e; }
-    }
-    best[k] = bv; bi[k] = bx;
-  }
-  float den = 0.f;
-  const float zmax = best[0];
-  for (int k = 0; k < top; ++k) { best[k] = expf(best[k] - zmax); den += best[k]; }
+  float w[32];
+  route_token<SCORING>(logits + (size_t)t * ldl, corr, cdt, E, top, bi, w);
   for (int k = 0; k < top; ++k) {
     ids[(size_t)t * top + k] = bi[k];
-    wts[(size_t)t * top + k] = best[k] / den;
+    wts[(size_t)t * top + k] = w[k];
+  }
+}
+
+// Few pairs (T * top <= 1024, E <= 256; decoding): the choice, the counts and the places in ONE workgroup -- the same ids, weights
+// and row order as the three launches below.
+template <int SCORING>
+__global__ __launch_bounds__(256) void moe_route_small_kernel(const float* __restrict__ logits, long ldl, const void* __restrict__ corr, int cdt,
+                                                              int32_t* __restrict__ ids, float* __restrict__ wts, int32_t* __restrict__ counts,
+                                                              int32_t* __restrict__ seg, int32_t* __restrict__ src_row, int32_t* __restrict__ dst,
+                                                              int T, int E, int top) {
+  __shared__ int ids_s[1024];
+  __shared__ int cnt_s[256];
+  const int tid = threadIdx.x, R = T * top;
+  for (int t = tid; t < T; t += 256) {
+    int bi[32];
+    float w[32];
+    route_token<SCORING>(logits + (size_t)t * ldl, corr, cdt, E, top, bi, w);
+    for (int k = 0; k < top; ++k) {
+      ids[(size_t)t * top + k] = ids_s[t * top + k] = bi[k];
+      wts[(size_t)t * top + k] = w[k];
+    }
+  }
+  __syncthreads();
+  int c = 0;
+  if (tid < E) {
+    for (int r = 0; r < R; ++r) c += ids_s[r] == tid;
+    cnt_s[tid] = c;
+    counts[tid] = c;
+  }
+  __syncthreads();
+  if (tid < E) {
+    int pos = 0;
+    for (int x = 0; x < tid; ++x) pos += cnt_s[x];
+    seg[tid] = pos;
+    if (tid == E - 1) seg[E] = pos + c;
+    for (int r = 0; r < R; ++r)
+      if (ids_s[r] == tid) {
+        src_row[pos] = r / top;
+        dst[r] = pos;
+        ++pos;
+      }
   }
 }
 
@@ -156,8 +192,13 @@ int dihip_seq_moe_route(void* stream, const float* logits, long ldl, int32_t* id
                     ldl >= E, DIHIP_PARAM_ERROR, "moe_route: bad argument (at most 32 choices per token)");
   if (T == 0) return DIHIP_SUCCESS;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-  if (scoring == 1) hipLaunchKernelGGL(moe_route_scores_kernel, dim3((T + 255) / 256), dim3(256), 0, s, logits, ldl, correction, w_dtype, ids, wts, T, E, top);
-  else hipLaunchKernelGGL(moe_route_kernel, dim3((T + 255) / 256), dim3(256), 0, s, logits, ldl, ids, wts, T, E, top);
+  if ((long)T * top <= 1024 && E <= 256) {
+    if (scoring == 1) hipLaunchKernelGGL(moe_route_small_kernel<1>, dim3(1), dim3(256), 0, s, logits, ldl, correction, w_dtype, ids, wts, counts, seg, src_row, dst, T, E, top);
+    else hipLaunchKernelGGL(moe_route_small_kernel<0>, dim3(1), dim3(256), 0, s, logits, ldl, correction, w_dtype, ids, wts, counts, seg, src_row, dst, T, E, top);
+    return launch_status();
+  }
+  if (scoring == 1) hipLaunchKernelGGL(moe_route_kernel<1>, dim3((T + 255) / 256), dim3(256), 0, s, logits, ldl, correction, w_dtype, ids, wts, T, E, top);
+  else hipLaunchKernelGGL(moe_route_kernel<0>, dim3((T + 255) / 256), dim3(256), 0, s, logits, ldl, correction, w_dtype, ids, wts, T, E, top);
   hipLaunchKernelGGL(moe_count_kernel, dim3(E), dim3(256), 0, s, ids, T * top, counts);
   hipLaunchKernelGGL(moe_place_kernel, dim3(E), dim3(256), 0, s, ids, T * top, top, E, counts, seg, src_row, dst);
   return launch_status();

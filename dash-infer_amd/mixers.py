@@ -223,12 +223,13 @@ class GroupedQueryAttention:
         if ctx.math == so.MATH_BF16 and self.mc:
             o = so.gqa_attn_mc(a, ktable, vtable, ctx.tok_pos, ctx.ent_slot, ctx.ent_row0, ctx.ent_count, ctx.max_count, ctx.max_pos,
                                H, G, D, V, self.scale, self.sink, self.sink_mode, self.softcap, gate, maps=self.maps, window=self.window,
-                               keep_first=self.keep_first)
+                               keep_first=self.keep_first,
+                               diff=(*self.differential, ctx.eps, ctx.act_buffer(H * V)) if self.differential is not None else None)
         else:
             o = so.gqa_attn(a, ktable, vtable, ctx.tok_slot, ctx.tok_pos, H, G, D, V, self.scale, self.sink, self.sink_mode,
                             self.softcap, gate, maps=self.maps, window=self.window, keep_first=self.keep_first)
-        if self.differential is not None:
-            o = so.maps_diff_norm(o, self.differential[0], self.differential[1], ctx.eps, H, V, out=ctx.act_buffer(H * V))
+            if self.differential is not None:
+                o = so.maps_diff_norm(o, self.differential[0], self.differential[1], ctx.eps, H, V, out=ctx.act_buffer(H * V))
         return so.linear(o, self.o, self.o_b, math=ctx.math)
 
 

@@ -46,7 +46,7 @@ _SIGS = {
     "dihip_gqa_attn_mc_supported": (i32, [i32, i32, i32, i32]),
     "dihip_gqa_attn_mc_workspace_bytes": (sz, [i32, i32, i32, i32]),
     "dihip_gqa_attn_mc": (i32, [vp, vp, lng, vp, lng, vp, vp, i32, i32, vp, i32, i32, f32, vp, lng, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32,
-                                i32, f32, i32, i32, i32, i32, vp, sz]),
+                                i32, f32, i32, i32, i32, i32, vp, sz, vp, i32, lng, f32, f32, f32]),
     "dihip_gla_workspace_bytes": (sz, [i32, i32, i32, i32, i32, i32, i32]),
     "dihip_gla": (i32, [vp, vp, lng, vp, lng, vp, lng, vp, lng, vp, lng, f32, f32, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, vp, sz]),
     "dihip_head_rmsnorm_mul": (i32, [vp, vp, i32, lng, vp, lng, vp, i32, f32, vp, lng, i32, i32, i32]),

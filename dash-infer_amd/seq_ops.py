@@ -261,8 +261,10 @@ def gqa_attn_mc_supported(D, DV, table):
 
 
 def gqa_attn_mc(q, ktable, vtable, tok_pos, ent_slot, ent_row0, ent_count, max_count, max_pos, H, G, D, DV, scale, sink=None,
-                sink_mode=SINK_NONE, softcap=0.0, gate=None, out=None, nsplit=None, maps=1, window=0, keep_first=0):
-    """the matrix-core form (bf16 pages); max_count / max_pos: the largest portion and position of the step (host numbers)"""
+                sink_mode=SINK_NONE, softcap=0.0, gate=None, out=None, nsplit=None, maps=1, window=0, keep_first=0, diff=None):
+    """the matrix-core form (bf16 pages); max_count / max_pos: the largest portion and position of the step (host numbers).
+    diff = (lam, out_scale, eps, y): with two maps, y [T, H * DV] <- maps_diff_norm of the result (inside the merge of a split walk)
+    and y is returned"""
     T, E = q.shape[0], ent_slot.shape[0]
     window, keep_first = int(window or 0), int(keep_first or 0)
     o = out if out is not None else torch.empty(T, H * maps * DV, dtype=torch.float32, device=q.device)
@@ -277,8 +279,10 @@ def gqa_attn_mc(q, ktable, vtable, tok_pos, ent_slot, ent_row0, ent_count, max_c
                                   ktable.span_len, ptr(sink), dt(sink) if sink is not None else F32_CODE, int(sink_mode), float(softcap or 0.0),
                                   ptr(gate), _rows(gate) if gate is not None else 0, ptr(tok_pos), ptr(ent_slot), ptr(ent_row0), ptr(ent_count),
                                   E, int(max_count), T, H, G, D, DV, float(scale), int(maps), window, keep_first, int(nsplit), ptr(ws),
-                                  ws.numel() if ws is not None else 0), "dihip_gqa_attn_mc")
-    return o
+                                  ws.numel() if ws is not None else 0, ptr(diff[3]) if diff else None, dt(diff[3]) if diff else F32_CODE,
+                                  _rows(diff[3]) if diff else 0, float(diff[0]) if diff else 0.0, float(diff[1]) if diff else 0.0,
+                                  float(diff[2]) if diff else 0.0), "dihip_gqa_attn_mc")
+    return diff[3] if diff else o
 
 
 def maps_diff_norm(x, lam, out_scale, eps, H, DV, out=None):

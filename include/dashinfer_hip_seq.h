@@ -80,14 +80,17 @@ int dihip_gqa_attn(void* stream, float* out, long ldo, const float* q, long ldq,
                    const float* gate, long ldg, const int32_t* tok_slot, const int32_t* tok_pos, int T, int H, int G, int D,
                    int DV, float scale, int maps, int window, int keep_first);
 /* the same on the matrix cores for bf16 pages (D, DV multiples of 8 up to 256 / 128, span_len a multiple of 32): rows given
- * as portions, the key walk split over nsplit workgroups (see dihip_latent_window_attn_mc) */
+ * as portions, the key walk split over nsplit workgroups (see dihip_latent_window_attn_mc).  diff_out != NULL (maps == 2):
+ * dihip_maps_diff_norm of the result goes to diff_out [T, H, DV] (rows of ldd elements of diff_dtype) -- inside the merge of a
+ * split walk, else as a launch of its own; `out` is then scratch. */
 int dihip_gqa_attn_mc_supported(int D, int DV, int span_len, int cache_dtype);
 size_t dihip_gqa_attn_mc_workspace_bytes(int T, int H_times_maps, int DV, int nsplit);
 int dihip_gqa_attn_mc(void* stream, float* out, long ldo, const float* q, long ldq, void* const* kspans, void* const* vspans,
                       int span_stride, int span_len, const void* sink, int w_dtype, int sink_mode, float softcap,
                       const float* gate, long ldg, const int32_t* tok_pos, const int32_t* ent_slot, const int32_t* ent_row0,
                       const int32_t* ent_count, int E, int max_count, int T, int H, int G, int D, int DV, float scale,
-                      int maps, int window, int keep_first, int nsplit, void* ws, size_t ws_bytes);
+                      int maps, int window, int keep_first, int nsplit, void* ws, size_t ws_bytes, void* diff_out, int diff_dtype,
+                      long ldd, float lam, float out_scale, float eps);
 /* two maps per head -> one (differential attention):  d = x[t, h, 0] - lam * x[t, h, 1];
  *   y[t, h, :] = d / sqrt(mean(d^2) + eps) * out_scale        x f32 [T, H, 2, DV], y [T, H, DV] of y_dtype */
 int dihip_maps_diff_norm(void* stream, void* y, int y_dtype, long ldy, const float* x, long ldx, float lam, float out_scale,
