@@ -7,6 +7,8 @@
 // 64 rows that run side by side: (1) every chunk composes its rows from S = 0 -> (product of its decays, the state it would end in), (2) the states the chunks really start from
 // are carried over the chunks, (3) every chunk runs its rows from that state and writes the outputs.
 // Beside it: the unit-RMS norm of every head's output times a multiplier (the output gate).
+// The same state kernels serve a state-space mixer with one scalar decay per head (dihip_ssd): its rows kernel writes the records
+//   decay = exp(-exp(a_log[h]) * dt) for every channel,  key = dt * B[group],  query = C[group],  dt = softplus(dt_raw + dt_bias[h]).
 #include "seq_common.h"
 
 namespace dihip {
@@ -40,6 +42,26 @@ __global__ __launch_bounds__(256) void gla_rows_kernel(GlaArgs a) {
       av = expf(log_sigmoid(a.z[(size_t)t * a.ldz + col]) * a.inv_tau);
       kv = a.k[(size_t)t * a.ldk + col];
       qv = a.q[(size_t)t * a.ldq + col] * a.q_scale;
+    }
+    float* r = a.rec + ((size_t)t * a.H + h) * 3 * a.Dp + i;
+    r[0] = av; r[a.Dp] = kv; r[2 * a.Dp] = qv;
+  }
+}
+
+// The records of a state-space mixer: B and C [T, G * D] are shared by the heads of a group (head h reads group h / (H / G)).
+__global__ __launch_bounds__(256) void ssd_rows_kernel(GlaArgs a, const float* __restrict__ dt, long lddt, const void* __restrict__ dt_bias,
+                                                       const void* __restrict__ a_log, int wdt, int G) {
+  const int t = blockIdx.x, hpg = a.H / G;
+  for (int c = threadIdx.x; c < a.H * a.Dp; c += 256) {
+    const int h = c / a.Dp, i = c - h * a.Dp;
+    float av = 1.f, kv = 0.f, qv = 0.f;
+    if (i < a.D) {
+      const float x = dt[(size_t)t * lddt + h] + ld_any(dt_bias, h, wdt);
+      const float step = x > 20.f ? x : log1pf(expf(x));
+      const size_t col = (size_t)(h / hpg) * a.D + i;
+      av = expf(-expf(ld_any(a_log, h, wdt)) * step);
+      kv = step * a.k[(size_t)t * a.ldk + col];
+      qv = a.q[(size_t)t * a.ldq + col];
     }
     float* r = a.rec + ((size_t)t * a.H + h) * 3 * a.Dp + i;
     r[0] = av; r[a.Dp] = kv; r[2 * a.Dp] = qv;
@@ -217,6 +239,30 @@ extern "C" {
 
 static int gla_dpad(int D) { return D <= 64 ? 64 : (D <= 128 ? 128 : 256); }
 
+// the state kernels over records that a rows kernel has written
+static void gla_launch_state(hipStream_t s, const GlaArgs& a, int E, int chunked, int cpt, int cbs) {
+  const int H = a.H, D = a.D, DV = a.DV, chunks = a.max_chunks;
+  const dim3 grid(chunks, H * cbs, E);
+  // four slices of Dp / 4 channels; two columns per thread where the registers allow (D <= 128)
+  auto go = [&](auto dpt, auto cp, auto ns) {
+    constexpr int DPT = decltype(dpt)::value, CPT = decltype(cp)::value, NS = decltype(ns)::value;
+    const dim3 block(64 * NS);
+    if (!chunked) {
+      hipLaunchKernelGGL((gla_kernel<DPT, 0, CPT, NS>), grid, block, 0, s, a);
+    } else {
+      hipLaunchKernelGGL((gla_kernel<DPT, 1, CPT, NS>), grid, block, 0, s, a);
+      hipLaunchKernelGGL(gla_carry_kernel, dim3((D * DV + 255) / 256, H, E), dim3(256), 0, s, a);
+      hipLaunchKernelGGL((gla_kernel<DPT, 3, CPT, NS>), grid, block, 0, s, a);
+    }
+  };
+  using one = std::integral_constant<int, 1>;
+  using two = std::integral_constant<int, 2>;
+  using four = std::integral_constant<int, 4>;
+  if (D <= 64) { if (cpt == 2) go(std::integral_constant<int, 16>{}, two{}, four{}); else go(std::integral_constant<int, 16>{}, one{}, four{}); }
+  else if (D <= 128) { if (cpt == 2) go(std::integral_constant<int, 32>{}, two{}, four{}); else go(std::integral_constant<int, 32>{}, one{}, four{}); }
+  else go(std::integral_constant<int, 64>{}, one{}, four{});
+}
+
 size_t dihip_gla_workspace_bytes(int T, int E, int max_count, int H, int D, int DV, int chunked) {
   size_t b = (size_t)T * H * 3 * gla_dpad(D) * sizeof(float);
   if (chunked) b += (size_t)E * ((max_count + GLA_CHUNK - 1) / GLA_CHUNK) * H * ((size_t)D * DV + D) * sizeof(float);
@@ -243,25 +289,31 @@ int dihip_gla(void* stream, float* out, long ldo, const float* q, long ldq, cons
   GlaArgs a{out, ldo, q, ldq, k, ldk, v, ldv, z, ldz, q_scale, 1.f / tau, state, ent_slot, ent_row0, ent_count, H, D, DV, Dp, T,
             rec, rec + (size_t)T * H * 3 * Dp, chunks};
   hipLaunchKernelGGL(gla_rows_kernel, dim3(T), dim3(256), 0, s, a);
-  const dim3 grid(chunks, H * cbs, E);
-  // four slices of Dp / 4 channels; two columns per thread where the registers allow (D <= 128)
-  auto go = [&](auto dpt, auto cp, auto ns) {
-    constexpr int DPT = decltype(dpt)::value, CPT = decltype(cp)::value, NS = decltype(ns)::value;
-    const dim3 block(64 * NS);
-    if (!chunked) {
-      hipLaunchKernelGGL((gla_kernel<DPT, 0, CPT, NS>), grid, block, 0, s, a);
-    } else {
-      hipLaunchKernelGGL((gla_kernel<DPT, 1, CPT, NS>), grid, block, 0, s, a);
-      hipLaunchKernelGGL(gla_carry_kernel, dim3((D * DV + 255) / 256, H, E), dim3(256), 0, s, a);
-      hipLaunchKernelGGL((gla_kernel<DPT, 3, CPT, NS>), grid, block, 0, s, a);
-    }
-  };
-  using one = std::integral_constant<int, 1>;
-  using two = std::integral_constant<int, 2>;
-  using four = std::integral_constant<int, 4>;
-  if (D <= 64) { if (cpt == 2) go(std::integral_constant<int, 16>{}, two{}, four{}); else go(std::integral_constant<int, 16>{}, one{}, four{}); }
-  else if (D <= 128) { if (cpt == 2) go(std::integral_constant<int, 32>{}, two{}, four{}); else go(std::integral_constant<int, 32>{}, one{}, four{}); }
-  else go(std::integral_constant<int, 64>{}, one{}, four{});
+  gla_launch_state(s, a, E, chunked, cpt, cbs);
+  return launch_status();
+}
+
+int dihip_ssd(void* stream, float* out, long ldo, const float* x, long ldx, const float* B, long ldb, const float* Cq, long ldc, const float* dt,
+              long lddt, const void* dt_bias, const void* a_log, int w_dtype, float* state, const int32_t* ent_slot, const int32_t* ent_row0,
+              const int32_t* ent_count, int T, int E, int max_count, int H, int G, int D, int DV, int chunked, void* ws, size_t ws_bytes) {
+  DIHIP_REQUIRE(T >= 0 && E >= 0 && max_count >= 0 && H > 0 && G > 0 && H % G == 0 && D > 0 && DV > 0 && out && x && B && Cq && dt && dt_bias &&
+                    a_log && state && ent_slot && ent_row0 && ent_count && ldo >= (long)H * DV && ldx >= (long)H * DV && ldb >= (long)G * D &&
+                    ldc >= (long)G * D && lddt >= H && seq_dtype_ok(w_dtype), DIHIP_PARAM_ERROR, "ssd: bad argument");
+  DIHIP_REQUIRE(D <= 256, DIHIP_EXCEED_LIMIT_ERROR, "ssd: more than 256 state channels per head (%d)", D);
+  const int cpt = (DV > 64 && D <= 128) ? 2 : 1;
+  const int cbs = (DV + 64 * cpt - 1) / (64 * cpt);
+  DIHIP_REQUIRE((long)H * cbs <= 65535 && E <= 65535, DIHIP_PARAM_ERROR, "ssd: too many heads or portions for one launch");
+  DIHIP_REQUIRE(ws && ws_bytes >= dihip_gla_workspace_bytes(T, E, max_count, H, D, DV, chunked) && (reinterpret_cast<uintptr_t>(ws) & 3u) == 0,
+                DIHIP_PARAM_ERROR, "ssd: workspace too small");
+  if (T == 0 || E == 0 || max_count == 0) return DIHIP_SUCCESS;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  const int chunks = chunked ? (max_count + GLA_CHUNK - 1) / GLA_CHUNK : 1;
+  const int Dp = gla_dpad(D);
+  float* rec = (float*)ws;
+  GlaArgs a{out, ldo, Cq, ldc, B, ldb, x, ldx, nullptr, 0, 1.f, 1.f, state, ent_slot, ent_row0, ent_count, H, D, DV, Dp, T,
+            rec, rec + (size_t)T * H * 3 * Dp, chunks};
+  hipLaunchKernelGGL(ssd_rows_kernel, dim3(T), dim3(256), 0, s, a, dt, lddt, dt_bias, a_log, w_dtype, G);
+  gla_launch_state(s, a, E, chunked, cpt, cbs);
   return launch_status();
 }
 

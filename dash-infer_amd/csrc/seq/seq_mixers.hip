@@ -331,7 +331,7 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(float* __restrict__ ou
 __global__ __launch_bounds__(256) void causal_conv_state_kernel(float* __restrict__ u, long ldu, const float* __restrict__ x, long ldx,
                                                                 const void* __restrict__ w, const void* __restrict__ bias, int wdt,
                                                                 const float* __restrict__ tail, const int32_t* __restrict__ tok_slot,
-                                                                const int32_t* __restrict__ tok_off, int C, int taps) {
+                                                                const int32_t* __restrict__ tok_off, int C, int taps, int silu) {
   const int t = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
   if (c >= C) return;
   const int off = tok_off[t], nt = taps - 1;
@@ -343,6 +343,7 @@ __global__ __launch_bounds__(256) void causal_conv_state_kernel(float* __restric
     acc = __builtin_fmaf(ld_any(w, (size_t)c * taps + k, wdt), v, acc);
   }
   if (bias) acc += ld_any(bias, c, wdt);
+  if (silu) acc = acc / (1.f + expf(-acc));
   u[(size_t)t * ldu + c] = acc;
 }
 
@@ -620,12 +621,13 @@ int dihip_latent_window_attn(void* stream, float* out, long ldo, const float* q,
 }
 
 int dihip_causal_conv_state(void* stream, float* u, long ldu, const float* x, long ldx, const void* w, const void* bias, int w_dtype,
-                            const float* tail, const int32_t* tok_slot, const int32_t* tok_off, int T, int C, int taps) {
+                            const float* tail, const int32_t* tok_slot, const int32_t* tok_off, int T, int C, int taps, int act) {
   DIHIP_REQUIRE(T >= 0 && C > 0 && taps >= 1 && taps <= 16 && u && x && w && (tail || taps == 1) && tok_slot && tok_off && ldu >= C &&
-                    ldx >= C && seq_dtype_ok(w_dtype), DIHIP_PARAM_ERROR, "causal_conv_state: bad argument (1 <= taps <= 16)");
+                    ldx >= C && seq_dtype_ok(w_dtype) && (act == 0 || act == 5), DIHIP_PARAM_ERROR,
+                "causal_conv_state: bad argument (1 <= taps <= 16; activation none or silu)");
   if (T == 0) return DIHIP_SUCCESS;
   hipLaunchKernelGGL(causal_conv_state_kernel, dim3(T, (C + 255) / 256), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), u, ldu, x, ldx,
-                     w, bias, w_dtype, tail, tok_slot, tok_off, C, taps);
+                     w, bias, w_dtype, tail, tok_slot, tok_off, C, taps, act == 5);
   return launch_status();
 }
 

@@ -16,13 +16,31 @@ namespace {
 // scores = softmax over all E logits, the choice by score + correction, weights = the chosen scores over their sum.  (Every logit
 // is read a few times: E is small and the row stays in cache.)
 template <int SCORING>
-__device__ __forceinline__ void route_token(const float* __restrict__ z, const void* __restrict__ corr, int cdt, int E, int top, int (&bi)[32],
-                                            float (&w)[32]) {
+__device__ __forceinline__ void route_token(const float* __restrict__ z, const void* __restrict__ corr, int cdt, int E, int top, int ngroups,
+                                            int keep, int (&bi)[32], float (&w)[32]) {
   float zmax = -INFINITY, den = 1.f;
   if (SCORING == 1) {
     for (int e = 0; e < E; ++e) zmax = fmaxf(zmax, z[e]);
     den = 0.f;
     for (int e = 0; e < E; ++e) den += expf(z[e] - zmax);
+  }
+  // group-limited choice: the experts form ngroups equal groups of neighbours, a group counts by its best expert, and only the
+  // experts of the `keep` best groups (ties: the lower index) can be chosen
+  uint32_t open_groups = 0xffffffffu;
+  const int gsz = ngroups > 1 ? E / ngroups : E;
+  if (ngroups > 1 && keep < ngroups) {
+    open_groups = 0u;
+    for (int k = 0; k < keep; ++k) {
+      float bv = -INFINITY;
+      int bg = -1;
+      for (int g = 0; g < ngroups; ++g) {
+        if (open_groups >> g & 1u) continue;
+        float gv = -INFINITY;
+        for (int e = g * gsz; e < (g + 1) * gsz; ++e) gv = fmaxf(gv, SCORING == 1 ? expf(z[e] - zmax) / den : z[e]);
+        if (bg < 0 || gv > bv) { bv = gv; bg = g; }
+      }
+      open_groups |= 1u << bg;
+    }
   }
   float sum = 0.f;
   for (int k = 0; k < top; ++k) {
@@ -36,6 +54,7 @@ __device__ __forceinline__ void route_token(const float* __restrict__ z, const v
         sc = expf(v - zmax) / den;
         v = sc + (corr ? ld_any(corr, e, cdt) : 0.f);
       }
+      if (ngroups > 1 && !(open_groups >> (e / gsz) & 1u)) used = true;
       if (!used && (bx < 0 || v > bv)) { bv = v; bx = e; bs = sc; }
     }
     w[k] = bs; bi[k] = bx;
@@ -53,12 +72,12 @@ __device__ __forceinline__ void route_token(const float* __restrict__ z, const v
 
 template <int SCORING>
 __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits, long ldl, const void* __restrict__ corr, int cdt,
-                                                        int32_t* __restrict__ ids, float* __restrict__ wts, int T, int E, int top) {
+                                                        int32_t* __restrict__ ids, float* __restrict__ wts, int T, int E, int top, int ngroups, int keep) {
   const int t = blockIdx.x * 256 + threadIdx.x;
   if (t >= T) return;
   int bi[32];
   float w[32];
-  route_token<SCORING>(logits + (size_t)t * ldl, corr, cdt, E, top, bi, w);
+  route_token<SCORING>(logits + (size_t)t * ldl, corr, cdt, E, top, ngroups, keep, bi, w);
   for (int k = 0; k < top; ++k) {
     ids[(size_t)t * top + k] = bi[k];
     wts[(size_t)t * top + k] = w[k];
@@ -71,14 +90,14 @@ template <int SCORING>
 __global__ __launch_bounds__(256) void moe_route_small_kernel(const float* __restrict__ logits, long ldl, const void* __restrict__ corr, int cdt,
                                                               int32_t* __restrict__ ids, float* __restrict__ wts, int32_t* __restrict__ counts,
                                                               int32_t* __restrict__ seg, int32_t* __restrict__ src_row, int32_t* __restrict__ dst,
-                                                              int T, int E, int top) {
+                                                              int T, int E, int top, int ngroups, int keep) {
   __shared__ int ids_s[1024];
   __shared__ int cnt_s[256];
   const int tid = threadIdx.x, R = T * top;
   for (int t = tid; t < T; t += 256) {
     int bi[32];
     float w[32];
-    route_token<SCORING>(logits + (size_t)t * ldl, corr, cdt, E, top, bi, w);
+    route_token<SCORING>(logits + (size_t)t * ldl, corr, cdt, E, top, ngroups, keep, bi, w);
     for (int k = 0; k < top; ++k) {
       ids[(size_t)t * top + k] = ids_s[t * top + k] = bi[k];
       wts[(size_t)t * top + k] = w[k];
@@ -185,7 +204,9 @@ using namespace dihip;
 extern "C" {
 
 int dihip_seq_moe_route(void* stream, const float* logits, long ldl, int32_t* ids, float* wts, int32_t* counts, int32_t* seg, int32_t* src_row,
-                    int32_t* dst, int T, int E, int top, int scoring, const void* correction, int w_dtype) {
+                    int32_t* dst, int T, int E, int top, int scoring, const void* correction, int w_dtype, int ngroups, int keep) {
+  DIHIP_REQUIRE(ngroups >= 1 && ngroups <= 32 && E % ngroups == 0 && keep >= 1 && keep <= ngroups && (long)keep * (E / ngroups) >= top,
+                DIHIP_PARAM_ERROR, "moe_route: at most 32 equal groups, of which the kept ones must hold the choices");
   DIHIP_REQUIRE((scoring == 0 || scoring == 1) && (!correction || scoring == 1) && seq_dtype_ok(w_dtype), DIHIP_PARAM_ERROR,
                 "moe_route: unknown scoring (a correction goes with scoring 1)");
   DIHIP_REQUIRE(T >= 0 && E > 0 && top > 0 && top <= E && top <= 32 && E <= 65535 && logits && ids && wts && counts && seg && src_row && dst &&
@@ -193,12 +214,12 @@ int dihip_seq_moe_route(void* stream, const float* logits, long ldl, int32_t* id
   if (T == 0) return DIHIP_SUCCESS;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   if ((long)T * top <= 1024 && E <= 256) {
-    if (scoring == 1) hipLaunchKernelGGL(moe_route_small_kernel<1>, dim3(1), dim3(256), 0, s, logits, ldl, correction, w_dtype, ids, wts, counts, seg, src_row, dst, T, E, top);
-    else hipLaunchKernelGGL(moe_route_small_kernel<0>, dim3(1), dim3(256), 0, s, logits, ldl, correction, w_dtype, ids, wts, counts, seg, src_row, dst, T, E, top);
+    if (scoring == 1) hipLaunchKernelGGL(moe_route_small_kernel<1>, dim3(1), dim3(256), 0, s, logits, ldl, correction, w_dtype, ids, wts, counts, seg, src_row, dst, T, E, top, ngroups, keep);
+    else hipLaunchKernelGGL(moe_route_small_kernel<0>, dim3(1), dim3(256), 0, s, logits, ldl, correction, w_dtype, ids, wts, counts, seg, src_row, dst, T, E, top, ngroups, keep);
     return launch_status();
   }
-  if (scoring == 1) hipLaunchKernelGGL(moe_route_kernel<1>, dim3((T + 255) / 256), dim3(256), 0, s, logits, ldl, correction, w_dtype, ids, wts, T, E, top);
-  else hipLaunchKernelGGL(moe_route_kernel<0>, dim3((T + 255) / 256), dim3(256), 0, s, logits, ldl, correction, w_dtype, ids, wts, T, E, top);
+  if (scoring == 1) hipLaunchKernelGGL(moe_route_kernel<1>, dim3((T + 255) / 256), dim3(256), 0, s, logits, ldl, correction, w_dtype, ids, wts, T, E, top, ngroups, keep);
+  else hipLaunchKernelGGL(moe_route_kernel<0>, dim3((T + 255) / 256), dim3(256), 0, s, logits, ldl, correction, w_dtype, ids, wts, T, E, top, ngroups, keep);
   hipLaunchKernelGGL(moe_count_kernel, dim3(E), dim3(256), 0, s, ids, T * top, counts);
   hipLaunchKernelGGL(moe_place_kernel, dim3(E), dim3(256), 0, s, ids, T * top, top, E, counts, seg, src_row, dst);
   return launch_status();

@@ -48,4 +48,4 @@ def read_config(path):
 
 
 def _load_builtin():
-    from . import modanex, qwen2, tobilorn, vogusun  # noqa: F401  (registration on import)
+    from . import filipel, modanex, qwen2, tobilorn, vogusun  # noqa: F401  (registration on import)

@@ -32,7 +32,7 @@ _SIGS = {
     "dihip_latent_window_attn_mc_workspace_bytes": (sz, [i32, i32, i32, i32]),
     "dihip_latent_window_attn_mc": (i32, [vp, vp, lng, vp, lng, vp, i32, i32, vp, i32, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, f32, i32,
                                           vp, sz]),
-    "dihip_causal_conv_state": (i32, [vp, vp, lng, vp, lng, vp, vp, i32, vp, vp, vp, i32, i32, i32]),
+    "dihip_causal_conv_state": (i32, [vp, vp, lng, vp, lng, vp, vp, i32, vp, vp, vp, i32, i32, i32, i32]),
     "dihip_conv_tail_update": (i32, [vp, vp, vp, lng, vp, vp, vp, i32, i32, i32]),
     "dihip_gated_recurrence_chunked_workspace_bytes": (sz, [i32, i32, i32]),
     "dihip_gated_recurrence_chunked": (i32, [vp, vp, lng, vp, vp, lng, vp, lng, vp, lng, vp, i32, f32, vp, vp, vp, vp, i32, i32, i32, vp, sz]),
@@ -50,9 +50,18 @@ _SIGS = {
     "dihip_gla_workspace_bytes": (sz, [i32, i32, i32, i32, i32, i32, i32]),
     "dihip_gla": (i32, [vp, vp, lng, vp, lng, vp, lng, vp, lng, vp, lng, f32, f32, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, vp, sz]),
     "dihip_head_rmsnorm_mul": (i32, [vp, vp, i32, lng, vp, lng, vp, i32, f32, vp, lng, i32, i32, i32]),
-    "dihip_seq_moe_route": (i32, [vp, vp, lng, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, vp, i32]),
+    "dihip_seq_moe_route": (i32, [vp, vp, lng, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, vp, i32, i32, i32]),
     "dihip_seq_moe_glu": (i32, [vp, vp, i32, lng, vp, lng, i32, i32, f32, f32, i32]),
     "dihip_seq_moe_combine": (i32, [vp, vp, lng, vp, lng, vp, vp, i32, i32, i32, vp, i32, vp, i32, lng, vp, lng]),
+    "dihip_residual_layernorm": (i32, [vp, vp, vp, vp, lng, vp, lng, f32, vp, vp, vp, i32, f32, vp, i32, lng, i32, i32]),
+    "dihip_polynorm": (i32, [vp, vp, i32, lng, vp, lng, vp, i32, f32, i32, i32]),
+    "dihip_rmsnorm_pair": (i32, [vp, vp, lng, vp, lng, vp, vp, lng, vp, i32, f32, f32, i32, i32]),
+    "dihip_gate_group_rmsnorm": (i32, [vp, vp, i32, lng, vp, lng, vp, lng, vp, vp, lng, vp, i32, f32, i32, i32, i32, i32]),
+    "dihip_latent_rope_append": (i32, [vp, vp, i32, i32, i32, vp, lng, vp, i32, f32, i32, i32, i32, vp, vp, lng, vp, lng, i32, vp, vp, i32]),
+    "dihip_ssd": (i32, [vp, vp, lng, vp, lng, vp, lng, vp, lng, vp, lng, vp, vp, i32, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, i32, vp, sz]),
+    "dihip_talk_attn_workspace_bytes": (sz, [i32, i32, i32, i32]),
+    "dihip_talk_attn": (i32, [vp, vp, i32, lng, vp, lng, vp, vp, i32, i32, i32, vp, vp, i32, vp, lng, vp, vp, i32, i32, i32, i32, i32, f32, i32, i32,
+                              vp, sz]),
     "dihip_gated_recurrence": (i32, [vp, vp, lng, vp, vp, lng, vp, lng, vp, lng, vp, i32, f32, vp, vp, vp, vp, i32, i32]),
 }
 

@@ -158,12 +158,13 @@ def latent_window_attn_mc(q, table, sink, tok_pos, ent_slot, ent_row0, ent_count
     return o
 
 
-def causal_conv_state(x, w, bias, tail, tok_slot, tok_off, out=None):
+def causal_conv_state(x, w, bias, tail, tok_slot, tok_off, out=None, act=None):
+    """act: None or "silu" on the result"""
     T, Cn = x.shape
     taps = w.shape[1]
     u = out if out is not None else torch.empty(T, Cn, dtype=torch.float32, device=x.device)
     check(lib().dihip_causal_conv_state(stream(), ptr(u), _rows(u), ptr(x), _rows(x), ptr(w), ptr(bias), dt(w), ptr(tail), ptr(tok_slot),
-                                        ptr(tok_off), T, Cn, taps), "dihip_causal_conv_state")
+                                        ptr(tok_off), T, Cn, taps, ACT[act]), "dihip_causal_conv_state")
     return u
 
 
@@ -324,8 +325,9 @@ ROUTE_CHOSEN_SOFTMAX, ROUTE_SCORES = 0, 1      # weights = softmax over the chos
 UNIT_CLAMPED, UNIT_SILU = 0, 1
 
 
-def moe_route(logits, top, scoring=ROUTE_CHOSEN_SOFTMAX, correction=None):
-    """-> ids [T, top] i32, wts [T, top] f32, seg [E + 1], src_row [T * top], dst [T * top]"""
+def moe_route(logits, top, scoring=ROUTE_CHOSEN_SOFTMAX, correction=None, groups=(1, 1)):
+    """groups = (count, keep): only experts of the `keep` best of `count` equal groups of neighbours can be chosen
+    -> ids [T, top] i32, wts [T, top] f32, seg [E + 1], src_row [T * top], dst [T * top]"""
     T, E = logits.shape
     dev = logits.device
     ints = torch.empty(T * top * 3 + 2 * E + 1, dtype=torch.int32, device=dev)
@@ -334,8 +336,8 @@ def moe_route(logits, top, scoring=ROUTE_CHOSEN_SOFTMAX, correction=None):
     wts = torch.empty(T, top, dtype=torch.float32, device=dev)
     assert correction is None or (correction.shape == (E,) and correction.is_contiguous())
     check(lib().dihip_seq_moe_route(stream(), ptr(logits), _rows(logits), ptr(ids), ptr(wts), ptr(counts), ptr(seg), ptr(src_row), ptr(dst),
-                                    T, E, int(top), int(scoring), ptr(correction), dt(correction) if correction is not None else F32_CODE),
-          "dihip_seq_moe_route")
+                                    T, E, int(top), int(scoring), ptr(correction), dt(correction) if correction is not None else F32_CODE,
+                                    int(groups[0]), int(groups[1])), "dihip_seq_moe_route")
     return ids.view(T, top), wts, seg, src_row, dst
 
 
@@ -353,4 +355,99 @@ def moe_combine(rows, dst, wts, T, top, out=None, ids=None, n_real=0, own=None, 
     check(lib().dihip_seq_moe_combine(stream(), ptr(o), _rows(o), ptr(rows), _rows(rows), ptr(dst), ptr(wts), T, int(top), K, ptr(ids), int(n_real),
                                       ptr(own), dt(own) if own is not None else F32_CODE, _rows(own) if own is not None else 0, ptr(add),
                                       _rows(add) if add is not None else 0), "dihip_seq_moe_combine")
+    return o
+
+
+def residual_layernorm(x_in, w=None, a=None, b=None, mult=1.0, eps=1e-5, x_out=None, row_idx=None, bias=None, out_dtype=torch.float32):
+    """x_out = x_in + mult * (a + b);  h = layer_norm(x_out) * w (+ bias)  (mean and variance over the row) -> h (None without w).
+    row_idx: the norm of the chosen rows of x_in alone."""
+    K = x_in.shape[1]
+    M = x_in.shape[0] if row_idx is None else row_idx.shape[0]
+    assert x_in.is_contiguous() and x_in.dtype == torch.float32 and (x_out is None or x_out.is_contiguous())
+    assert a is None or x_out is not None
+    h = torch.empty(M, K, dtype=out_dtype, device=x_in.device) if w is not None else None
+    check(lib().dihip_residual_layernorm(stream(), ptr(x_out), ptr(x_in), ptr(a), _rows(a) if a is not None else 0, ptr(b),
+                                         _rows(b) if b is not None else 0, float(mult), ptr(row_idx), ptr(w), ptr(bias),
+                                         dt(w) if w is not None else F32_CODE, float(eps), ptr(h), dt(h) if h is not None else F32_CODE,
+                                         _rows(h) if h is not None else 0, M, K), "dihip_residual_layernorm")
+    return h
+
+
+def polynorm(z, coef, eps, out):
+    """out = c0 z / rms(z) + c1 z^2 / rms(z^2) + c2 z^3 / rms(z^3) + c3 over the rows of z (f32); coef: the four numbers"""
+    T, F = z.shape
+    assert z.dtype == torch.float32 and out.shape == (T, F) and coef.numel() == 4 and coef.is_contiguous()
+    check(lib().dihip_polynorm(stream(), ptr(out), dt(out), _rows(out), ptr(z), _rows(z), ptr(coef), dt(coef), float(eps), T, F), "dihip_polynorm")
+    return out
+
+
+def rmsnorm_pair(xa, wa, xb, wb, coef, eps, out=None):
+    """coef * (xa / rms(xa) * wa + xb / rms(xb) * wb) -> f32 [T, K]"""
+    T, K = xa.shape
+    assert xb.shape == (T, K) and xa.dtype == xb.dtype == torch.float32 and wa.dtype == wb.dtype and wa.shape[0] == wb.shape[0] == K
+    y = out if out is not None else torch.empty(T, K, dtype=torch.float32, device=xa.device)
+    check(lib().dihip_rmsnorm_pair(stream(), ptr(y), _rows(y), ptr(xa), _rows(xa), ptr(wa), ptr(xb), _rows(xb), ptr(wb), dt(wa), float(coef),
+                                   float(eps), T, K), "dihip_rmsnorm_pair")
+    return y
+
+
+def gate_group_rmsnorm(o, z, w, eps, heads, P, groups, x=None, skip=None, out=None):
+    """v = (o + skip[head] * x) * silu(z); out = v / rms(v over each of `groups` equal parts of the row) * w"""
+    T = o.shape[0]
+    y = out if out is not None else torch.empty(T, heads * P, dtype=torch.float32, device=o.device)
+    assert o.dtype == z.dtype == torch.float32 and w.shape[0] == heads * P and (skip is None or (skip.dtype == w.dtype and x is not None))
+    check(lib().dihip_gate_group_rmsnorm(stream(), ptr(y), dt(y), _rows(y), ptr(o), _rows(o), ptr(x), _rows(x) if x is not None else 0,
+                                         ptr(skip), ptr(z), _rows(z), ptr(w), dt(w), float(eps), T, int(heads), int(P), int(groups)),
+          "dihip_gate_group_rmsnorm")
+    return y
+
+
+def latent_rope_append(table, ckv, gamma, eps, R, rot, freq, q_rot, ql, H, tok_slot, tok_pos, append=True):
+    """table: the SpanTable of rows [R latent | rot key part | padding]; append False: only the queries' rotated parts are written
+    (a layer that reads another layer's pages)"""
+    T, Rp = ql.shape[0], table.row_elems
+    assert ql.dtype == q_rot.dtype == torch.float32 and ql.shape[1] == H * Rp and q_rot.shape[1] == H * rot
+    assert not append or (ckv.dtype == torch.float32 and ckv.shape[1] == R + rot)
+    check(lib().dihip_latent_rope_append(stream(), ptr(table.ptrs) if append else None, table.max_spans, table.span_len, _DT[table.dtype],
+                                         ptr(ckv) if append else None, _rows(ckv) if append else 0, ptr(gamma) if append else None,
+                                         dt(gamma) if append and gamma is not None else F32_CODE, float(eps), int(R), int(rot), int(Rp),
+                                         ptr(freq), ptr(q_rot), _rows(q_rot), ptr(ql), _rows(ql), int(H), ptr(tok_slot), ptr(tok_pos), T),
+          "dihip_latent_rope_append")
+
+
+def ssd(x, B, Cq, dtr, dt_bias, a_log, state, ent_slot, ent_row0, ent_count, max_count, H, G, D, DV, out=None, chunked=None):
+    """state-space scan with a scalar decay per head: x [T, >= H * DV], B / Cq [T, >= G * D], dtr [T, >= H] f32 rows; state
+    [slots, H, D, DV] f32 -> f32 [T, H * DV]"""
+    T, E = x.shape[0], ent_slot.shape[0]
+    assert state.shape[1:] == (H, D, DV) and state.is_contiguous() and dt_bias.dtype == a_log.dtype
+    o = out if out is not None else torch.empty(T, H * DV, dtype=torch.float32, device=x.device)
+    if chunked is None:
+        chunked = max_count >= CHUNKED_GLA_ROWS
+    chunked = 1 if chunked else 0
+    ws = torch.empty(int(lib().dihip_gla_workspace_bytes(T, E, int(max_count), H, D, DV, chunked)), dtype=torch.uint8, device=x.device)
+    check(lib().dihip_ssd(stream(), ptr(o), _rows(o), ptr(x), _rows(x), ptr(B), _rows(B), ptr(Cq), _rows(Cq), ptr(dtr), _rows(dtr), ptr(dt_bias),
+                          ptr(a_log), dt(a_log), ptr(state), ptr(ent_slot), ptr(ent_row0), ptr(ent_count), T, E, int(max_count), int(H), int(G),
+                          int(D), int(DV), chunked, ptr(ws), ws.numel()), "dihip_ssd")
+    return o
+
+
+TALK_MAX_HEADS = 64
+
+
+def talk_attn(q, ktable, vtable, tok_slot, tok_pos, max_pos, H, G, D, DV, scale, talk, temp=None, gate=None, window=0, out=None, nsplit=None):
+    """attention whose softmax maps are mixed between the heads (talk [H, H]) after the softmax; temp [H]: a multiplier per head on
+    the scores; gate: f32 [T, >= H * DV] multiplier.  max_pos: the step's last position (a host number: it sizes the split of the
+    key walk for few rows) -> [T, H * DV] (f32, or `out`)"""
+    T = q.shape[0]
+    window = int(window or 0)
+    o = out if out is not None else torch.empty(T, H * DV, dtype=torch.float32, device=q.device)
+    if nsplit is None:       # fill the chip: one workgroup per (row, part), at least 128 keys a part
+        keys = min(max_pos + 1, window) if window > 0 else max_pos + 1
+        nsplit = max(1, min(256 // max(T, 1), (keys + 127) // 128))
+    ws = torch.empty(int(lib().dihip_talk_attn_workspace_bytes(T, H, DV, nsplit)), dtype=torch.uint8, device=q.device)
+    assert talk.shape == (H, H) and talk.is_contiguous() and (temp is None or (temp.dtype == talk.dtype and temp.shape == (H,)))
+    check(lib().dihip_talk_attn(stream(), ptr(o), dt(o), _rows(o), ptr(q), _rows(q), ptr(ktable.ptrs), ptr(vtable.ptrs), ktable.max_spans,
+                                ktable.span_len, _DT[ktable.dtype], ptr(temp), ptr(talk), dt(talk), ptr(gate),
+                                _rows(gate) if gate is not None else 0, ptr(tok_slot), ptr(tok_pos), T, H, G, D, DV, float(scale), window,
+                                int(nsplit), ptr(ws), ws.numel()), "dihip_talk_attn")
     return o

@@ -56,6 +56,54 @@ int dihip_add_dyt(void* stream, float* x_out, const float* x_in, const float* a,
                   const int32_t* row_idx, float alpha, const void* w, const void* bias, int w_dtype, float* h, void* h16,
                   int M, int K);
 
+/* Layers that run their sublayers side by side on a layer-normed stream: the residual step and the NEXT input norm in one launch,
+ *   x_out[r] = x_in[r] + mult * (a[r] + b[r])   (a NULL: x_in itself; b NULL: a alone),
+ *   h[i] = (x_out[r] - mean) / sqrt(var + eps) * w (+ bias)   (mean and variance over the row; bias NULL: none; w NULL: no norm)
+ * r = row_idx ? row_idx[i] : i (with row_idx x_out must be NULL).  x_in / x_out: contiguous [., K] f32 (may alias); h: rows of
+ * stride ldh, f32 or bf16. */
+int dihip_residual_layernorm(void* stream, float* x_out, const float* x_in, const float* a, long lda, const float* b, long ldb,
+                             float mult, const int32_t* row_idx, const void* w, const void* bias, int w_dtype, float eps, void* h,
+                             int h_dtype, long ldh, int M, int K);
+/* y[t] = c0 z / rms(z) + c1 z^2 / rms(z^2) + c2 z^3 / rms(z^3) + c3,  powers per element, rms(v) = sqrt(mean(v^2) + eps) over the
+ * F elements of the row; coef = (c0, c1, c2, c3) of w_dtype */
+int dihip_polynorm(void* stream, void* y, int y_dtype, long ldy, const float* z, long ldz, const void* coef, int w_dtype, float eps,
+                   int T, int F);
+/* y[t] = coef * (xa[t] / rms(xa[t]) * wa + xb[t] / rms(xb[t]) * wb)   (wa, wb [K] of w_dtype) */
+int dihip_rmsnorm_pair(void* stream, float* y, long ldy, const float* xa, long lda, const void* wa, const float* xb, long ldb,
+                       const void* wb, int w_dtype, float coef, float eps, int T, int K);
+/* v = (o + skip[c / P] * x) * silu(z)  (skip [heads] or NULL);  y = v / rms(v over its part) * w,  the row of heads * P elements
+ * in `groups` equal parts, w [heads * P] */
+int dihip_gate_group_rmsnorm(void* stream, void* y, int y_dtype, long ldy, const float* o, long ldo, const float* x, long ldx,
+                             const void* skip, const float* z, long ldz, const void* w, int w_dtype, float eps, int T, int heads, int P,
+                             int groups);
+/* Attention through a latent with ONE rotated key part shared by the heads.  ckv[t] = [R latent | rot key part] (f32): the page
+ * row of the token (Rp elements) becomes [latent / rms * gamma | rotated key part | zeros]  (spans NULL: nothing is appended --
+ * a layer that reads another layer's pages).  q_rot[t] = [H][rot]: every head's rotated query part goes to ql[t][h * Rp + R ..]
+ * (behind the head's absorbed query).  Rotation: dimension i with i + rot / 2 by the angle float(pos) * freq[i]. */
+int dihip_latent_rope_append(void* stream, void* const* spans, int span_stride, int span_len, int cache_dtype, const float* ckv,
+                             long ldc, const void* gamma, int w_dtype, float eps, int R, int rot, int Rp, const float* freq,
+                             const float* q_rot, long ldqr, float* ql, long ldql, int H, const int32_t* tok_slot,
+                             const int32_t* tok_pos, int T);
+
+/* State-space mixer with a scalar decay per head and a matrix state [D, DV] per head and slot (the state kernels of dihip_gla):
+ *   step = softplus(dt[t, h] + dt_bias[h]);  S <- exp(-exp(a_log[h]) * step) S + step * B[t, g] x[t, h]^T;  out[t, h] = S^T C[t, g]
+ * g = h / (H / G).  x [T, H * DV], B / C [T, G * D], dt [T, H] f32 rows; workspace: dihip_gla_workspace_bytes. */
+int dihip_ssd(void* stream, float* out, long ldo, const float* x, long ldx, const float* B, long ldb, const float* Cq, long ldc,
+              const float* dt, long lddt, const void* dt_bias, const void* a_log, int w_dtype, float* state, const int32_t* ent_slot,
+              const int32_t* ent_row0, const int32_t* ent_count, int T, int E, int max_count, int H, int G, int D, int DV, int chunked,
+              void* ws, size_t ws_bytes);
+
+/* Grouped-query attention whose softmax maps are mixed between the heads after the softmax:
+ *   w_g(i, j) = softmax over the row's window of q_g(i) . k(j) * scale * temp[g];  out_h(i) = sum_j (sum_g talk[h, g] w_g(i, j)) v(j)
+ * q: f32 rows [H, D] (already rotated), keys [G, D] and values [G, DV] in their pages, head h reads key/value head h / (H / G);
+ * window <= 0: every key up to the row's own; temp [H] or NULL, talk [H, H] (w_dtype); gate: f32 [T, H * DV] multiplier or NULL;
+ * out: rows [H * DV] of out_dtype.  nsplit: parts of the key walk (a host choice); workspace: the statistics and the parts. */
+size_t dihip_talk_attn_workspace_bytes(int T, int H, int DV, int nsplit);
+int dihip_talk_attn(void* stream, void* out, int out_dtype, long ldo, const float* q, long ldq, void* const* kspans, void* const* vspans,
+                    int span_stride, int span_len, int cache_dtype, const void* temp, const void* talk, int w_dtype, const float* gate,
+                    long ldg, const int32_t* tok_slot, const int32_t* tok_pos, int T, int H, int G, int D, int DV, float scale,
+                    int window, int nsplit, void* ws, size_t ws_bytes);
+
 /* Grouped-query attention, step 1: per token the rows qkv[t] hold q [H, maps, D] at column q_off, k [G, maps, D] at k_off,
  * v [G, DV] at v_off (f32; maps = the softmax maps per head, 1 for ordinary attention).  Every query and key head is divided by its root mean square and scaled by qnorm / knorm [D] (NULL: no norm),
  * then rotated on its first rot_dims dimensions by the angles tok_pos[t] * freq[i] (f32 product; layout 0: dimension 2i
@@ -113,9 +161,12 @@ int dihip_head_rmsnorm_mul(void* stream, void* y, int y_dtype, long ldy, const f
 /* Mixture of experts: per token the `top` experts of largest logit (ties: the lower index) and the softmax over the chosen
  * logits (scoring 0), or scores = softmax over all E logits, the `top` experts of largest score + correction[e] (correction
  * [E] of w_dtype, NULL: none) and weights = their scores / (the sum of their scores + 1e-20) (scoring 1) -> ids / wts [T, top]; the T * top (token, choice) pairs grouped by expert -> seg [E + 1], src_row [T * top] (the
- * token a sorted row reads), dst [T * top] (the sorted row of pair t * top + k); counts: [E] scratch. */
+ * token a sorted row reads), dst [T * top] (the sorted row of pair t * top + k); counts: [E] scratch.
+ * ngroups > 1: the experts form ngroups equal groups of neighbours; a group counts by its largest score (scoring 1) or logit, and
+ * only experts of the `keep` best groups can be chosen (ngroups = keep = 1: no limit). */
 int dihip_seq_moe_route(void* stream, const float* logits, long ldl, int32_t* ids, float* wts, int32_t* counts, int32_t* seg,
-                    int32_t* src_row, int32_t* dst, int T, int E, int top, int scoring, const void* correction, int w_dtype);
+                    int32_t* src_row, int32_t* dst, int T, int E, int top, int scoring, const void* correction, int w_dtype,
+                    int ngroups, int keep);
 /* unit 0: y[r, c] = g * sigmoid(slope * g) * (u + 1),  g = min(gu[r, c], limit),  u = clamp(gu[r, F + c], -limit, limit)
  * unit 1: y[r, c] = silu(gu[r, c]) * gu[r, F + c] */
 int dihip_seq_moe_glu(void* stream, void* y, int y_dtype, long ldy, const float* gu, long ldgu, int R, int F, float limit,
@@ -187,10 +238,11 @@ int dihip_latent_window_attn_mc(void* stream, float* out, long ldo, const float*
                                 size_t ws_bytes);
 
 /* u[t, c] = bias[c] + sum_{k < taps} w[c, k] * src(t, k),  src = x[t - (taps - 1 - k), c] inside the portion, else the
- * slot's tail state [slots][taps - 1][C] f32 (the last taps - 1 inputs of the sequence; zeros at its start) */
+ * slot's tail state [slots][taps - 1][C] f32 (the last taps - 1 inputs of the sequence; zeros at its start); act: 0, or 5 for
+ * silu on the result */
 int dihip_causal_conv_state(void* stream, float* u, long ldu, const float* x, long ldx, const void* w,
                             const void* bias, int w_dtype, const float* tail, const int32_t* tok_slot,
-                            const int32_t* tok_off, int T, int C, int taps);
+                            const int32_t* tok_off, int T, int C, int taps, int act);
 /* after it: tail <- the last taps - 1 inputs of every portion (ent_slot / ent_row0 / ent_count: [E]) */
 int dihip_conv_tail_update(void* stream, float* tail, const float* x, long ldx, const int32_t* ent_slot,
                            const int32_t* ent_row0, const int32_t* ent_count, int E, int C, int taps);
