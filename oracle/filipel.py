@@ -221,3 +221,116 @@ def forward(cfg, tensors, tokens, streams=None):
         if streams is not None:
             streams.append(x.copy())
     return layer_norm(x, tensors["final.norm"], eps) @ f64(tensors["head"]).T
+
+
+# -- small random models (tests) --------------------------------------------------------------------------------------------
+def bf16_values(a):
+    """float32 array whose values are exactly representable in bfloat16 (round to nearest even)"""
+    u = np.asarray(a, np.float32).view(np.uint32)
+    u = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16) << 16
+    return u.astype(np.uint32).view(np.float32)
+
+
+LEFT = dict(heads=6, kv_heads=2, dim=16, vdim=24, window=40, rot_dims=8, base=10000.0, scale=None)
+RIGHT = dict(heads=3, vdim=20, state=12, groups=1, conv=3, norm_groups=2)
+LATENT = dict(heads=3, dim=16, rot_dim=8, vdim=20, kv_rank=24, q_rank=28, base=5000.0, scale=None, kv_from=None)
+MOE = dict(experts=6, count=3, keep=2, top=2, ff=20)
+
+
+def left_weights(rng, width, o):
+    bf = bf16_values
+    r = lambda *s: bf(rng.normal(0, 1.0 / math.sqrt(s[-1]), s))
+    H, G, D, V = o["heads"], o["kv_heads"], o["dim"], o["vdim"]
+    return {"q": r(H * D, width), "k": r(G * D, width), "v": r(G * V, width), "g": r(H * V, width), "o": r(width, H * V),
+            "talk": bf(np.eye(H) * 0.8 + 0.3 * rng.normal(size=(H, H))), "temp": bf(rng.uniform(0.6, 1.6, H)),
+            "out": bf(1.0 + 0.2 * rng.normal(size=width))}
+
+
+def left_config(o):
+    return {"heads": o["heads"], "kv_heads": o["kv_heads"], "dim": o["dim"], "vdim": o["vdim"], "mask": {"size": o["window"]},
+            "rot": {"base": o["base"], "dims": o["rot_dims"]}, "scale": o["scale"] if o["scale"] is not None else o["dim"] ** -0.5}
+
+
+def right_weights(rng, width, o):
+    bf = bf16_values
+    r = lambda *s: bf(rng.normal(0, 1.0 / math.sqrt(s[-1]), s))
+    Hn, P, N, G, taps = o["heads"], o["vdim"], o["state"], o["groups"], o["conv"]
+    inner, ch = Hn * P, Hn * P + 2 * G * N
+    return {"in": r(2 * inner + 2 * G * N + Hn, width), "conv": bf(rng.normal(0, 0.6, (ch, taps))), "conv.b": bf(0.1 * rng.normal(size=ch)),
+            "dt_bias": bf(rng.uniform(-3.0, 0.5, Hn)), "A_log": bf(np.log(rng.uniform(0.3, 4.0, Hn))), "D": bf(rng.normal(size=Hn)),
+            "norm": bf(1.0 + 0.2 * rng.normal(size=inner)), "o": r(width, inner), "out": bf(1.0 + 0.2 * rng.normal(size=width))}
+
+
+def right_config(o):
+    return {k: o[k] for k in ("heads", "vdim", "state", "groups", "conv", "norm_groups")}
+
+
+def latent_weights(rng, width, o):
+    bf = bf16_values
+    r = lambda *s: bf(rng.normal(0, 1.0 / math.sqrt(s[-1]), s))
+    H, D, Rd, V, R, Q = o["heads"], o["dim"], o["rot_dim"], o["vdim"], o["kv_rank"], o["q_rank"]
+    w = {"dq": r(Q, width), "dq.norm": bf(1.0 + 0.2 * rng.normal(size=Q)), "uq": r(H * (D + Rd), Q), "uk": r(H * D, R), "uv": r(H * V, R),
+         "g": r(H * V, width), "o": r(width, H * V)}
+    if o.get("kv_from") is None:
+        w["dkv"], w["dkv.norm"] = r(R + Rd, width), bf(1.0 + 0.2 * rng.normal(size=R))
+    return w
+
+
+def latent_config(o):
+    m = {"heads": o["heads"], "dim": o["dim"], "rot_dim": o["rot_dim"], "vdim": o["vdim"], "kv_rank": o["kv_rank"], "q_rank": o["q_rank"],
+         "rot": {"base": o["base"], "dims": o["rot_dim"]}, "scale": o["scale"] if o["scale"] is not None else (o["dim"] + o["rot_dim"]) ** -0.5}
+    if o.get("kv_from") is not None:
+        m["kv_from"] = o["kv_from"]
+    return m
+
+
+def ff_weights(rng, width, fc):
+    bf = bf16_values
+    r = lambda *s: bf(rng.normal(0, 1.0 / math.sqrt(s[-1]), s))
+    if fc["kind"] == "dense":
+        return {"up": r(fc["ff"], width), "down": r(width, fc["ff"]), "act": bf(np.array([0.7, 0.35, -0.2, 0.05]) + 0.05 * rng.normal(size=4))}
+    w = {"router": bf(rng.normal(0, 2.0 / math.sqrt(width), (fc["router"]["experts"], width)))}
+    for e in range(fc["router"]["experts"]):
+        w[f"e{e}.gate"], w[f"e{e}.up"], w[f"e{e}.down"] = r(fc["expert"]["ff"], width), r(fc["expert"]["ff"], width), r(width, fc["expert"]["ff"])
+    return w
+
+
+def ff_config(spec):
+    """spec: None, ("dense", ff) or ("moe", overrides of MOE)"""
+    if spec is None:
+        return None
+    if spec[0] == "dense":
+        return {"kind": "dense", "ff": int(spec[1])}
+    o = dict(MOE, **(spec[1] if len(spec) > 1 else {}))
+    return {"kind": "moe", "expert": {"ff": o["ff"]}, "router": {"experts": o["experts"], "top": o["top"], "groups": {"count": o["count"], "keep": o["keep"]}}}
+
+
+def random_filipel(rng, layers, width=72, vocab=97, eps=1e-5, residual_mult=0.5):
+    """A small random model -> (config, tensors as float32 arrays of bf16 values).  layers: a list of (type, mixer overrides, ff spec):
+    type "parallel" with overrides {"left": {..}, "right": {..}} of LEFT / RIGHT, or "latent_attention" with overrides of LATENT;
+    ff spec as ff_config takes it."""
+    bf = bf16_values
+    cfg = {"architecture": "Filipel", "width": width, "vocab": vocab, "norm": {"eps": eps}, "residual_mult": residual_mult, "layers": []}
+    t = {"embed": bf(rng.normal(size=(vocab, width))), "head": bf(rng.normal(0, 1.0 / math.sqrt(width), (vocab, width))),
+         "final.norm": bf(1.0 + 0.2 * rng.normal(size=width))}
+    for i, (kind, over, ff) in enumerate(layers):
+        p = f"l{i}."
+        t[p + "norm1"] = bf(1.0 + 0.2 * rng.normal(size=width))
+        if kind == "parallel":
+            lo, ro = dict(LEFT, **(over or {}).get("left", {})), dict(RIGHT, **(over or {}).get("right", {}))
+            m = {"left": left_config(lo), "right": right_config(ro)}
+            for k, v in left_weights(rng, width, lo).items():
+                t[p + "mix.left." + k] = v
+            for k, v in right_weights(rng, width, ro).items():
+                t[p + "mix.right." + k] = v
+        else:
+            o = dict(LATENT, **(over or {}))
+            m = latent_config(o)
+            for k, v in latent_weights(rng, width, o).items():
+                t[p + "mix." + k] = v
+        fc = ff_config(ff)
+        if fc is not None:
+            for k, v in ff_weights(rng, width, fc).items():
+                t[p + "mlp." + k] = v
+        cfg["layers"].append({"type": kind, "mixer": m, "mlp": fc})
+    return cfg, t
