@@ -1031,7 +1031,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=8)
-    ap.add_argument("--workload", default="int4_b1", choices=list(WORKLOADS) + ["launch_selftest", "modanex_layers", "vogusun_layers", "tobilorn_layers"])  # int4_b1 = the headline configuration
+    ap.add_argument("--workload", default="int4_b1", choices=list(WORKLOADS) + ["launch_selftest", "modanex_layers", "vogusun_layers", "tobilorn_layers", "filipel_layers"])  # int4_b1 = the headline configuration
     ap.add_argument("--layers", type=int, default=None, help="debug: fewer decoder layers (result marked invalid)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="debug: eager launches instead of hipGraph replay")
@@ -1112,6 +1112,16 @@ def main():
         out = tobilorn_bench.run(args)
         os.makedirs(os.path.join(ROOT, "gpurun_out"), exist_ok=True)
         with open(os.path.join(ROOT, "gpurun_out", "bench_tobilorn_layers.json"), "w") as f:
+            json.dump(out, f, indent=1)
+        print(json.dumps(out), flush=True)
+        return
+    if args.workload == "filipel_layers":
+        # the sequence engine on random Filipel models of real layer sizes, beside Vogusun models of equal size (dash-infer_amd/filipel_bench.py)
+        assert world == 1, "filipel_layers is a one-GPU workload"
+        from dash_infer_amd import filipel_bench
+        out = filipel_bench.run(args)
+        os.makedirs(os.path.join(ROOT, "gpurun_out"), exist_ok=True)
+        with open(os.path.join(ROOT, "gpurun_out", "bench_filipel_layers.json"), "w") as f:
             json.dump(out, f, indent=1)
         print(json.dumps(out), flush=True)
         return

@@ -190,6 +190,209 @@ __global__ __launch_bounds__(256) void talk_merge_kernel(TalkArgs a) {
   }
 }
 
+
+// ------------------------------------------------------------------------------------------------ matrix-core kernel (bf16 pages)
+// A workgroup of 8 waves owns 16 consecutive rows of ONE portion and EVERY head, and walks the 16-key tiles those rows can see, the
+// tile's keys (pass 2: and values) of all key/value heads staged in LDS.  Per tile every wave scores HPW heads on the matrix cores
+// (S^T = K . Q^T, the query fragments held in registers); lane (row, kb) then holds the keys kb * 4 .. + 3 of its row.
+//   PASS 1: the running maximum and denominator of every (row, head) -> stats.
+//   PASS 2: the normalised weights of all heads go to LDS ([head][row][key] f32); after a barrier a wave mixes, for each of its OPW
+//           output heads, the weights of all heads at its lane's four keys (f32, the mixing row through scalar loads), packs them
+//           to bf16 and adds O^T += V^T . P^T on the matrix cores (V^T through the transposing LDS read).
+// Scoring every head is cheap beside the mix, so with many heads gridDim.z workgroups share a row tile: each scores all heads and
+// owns a part of the OUTPUT heads (fewer accumulators per wave).
+typedef short bf16x4s_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ f32x4_t mfma_bf16t(const u32x4_t& a, const u32x4_t& b, const f32x4_t& c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+}
+__device__ __forceinline__ f32x4_t mfma_bf16k16(const u32x2_t& a, const u32x2_t& b, const f32x4_t& c) {
+  return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(bf16x4s_t, a), __builtin_bit_cast(bf16x4s_t, b), c, 0, 0, 0);
+}
+typedef const __attribute__((address_space(4))) float* talk_uniform_ptr;   // read-only for the launch, wave-uniform address: scalar loads
+
+struct TalkMcArgs {
+  void* out; int odt; long ldo;
+  const float* q; long ldq;
+  void* const* kspans; void* const* vspans; int span_stride, span_len;
+  const void* temp; int wdt; const float* talk32;   // temp [H] (NULL: 1); talk32: f32 [H][H]
+  const float* gate; long ldg;
+  const int32_t* tok_pos; const int32_t* ent_slot; const int32_t* ent_row0; const int32_t* ent_count;
+  int H, G, D, DV; float scale; int window;
+  float* stats;                                     // [T][H][2]
+};
+
+template <int PASS, int HPW, int OPW, int DMAX, int VMAX>
+__global__ __launch_bounds__(512) void talk_attn_mc_kernel(TalkMcArgs a) {
+  constexpr int KS = DMAX / 32, DT = VMAX / 16;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  const int G = a.G, H = a.H, D = a.D, DV = a.DV, hpg = H / G;
+  const int e = blockIdx.y, cnt = a.ent_count[e], row0 = a.ent_row0[e];
+  const int r0 = blockIdx.x * 16;
+  if (r0 >= cnt) return;
+  const int tid = threadIdx.x, lane = tid & 63, ni = lane & 15, kb = lane >> 4;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int pitchk = (D + 8) * 2, pitchv = (DV + 8) * 2;
+  unsigned char* ksm = smem;                                   // [G][16][pitchk]
+  unsigned char* vsm = ksm + G * 16 * pitchk;                  // [G][16][pitchv]   (PASS 2)
+  float* psm = reinterpret_cast<float*>(vsm + (PASS == 2 ? G * 16 * pitchv : 0));   // [H][16 rows][16 keys]   (PASS 2)
+  const int pos0 = a.tok_pos[row0];
+  const bool row_ok = r0 + ni < cnt;
+  const int tq = min(r0 + ni, cnt - 1), p = pos0 + tq;
+  const int p_lo = pos0 + r0, p_hi = pos0 + min(r0 + 15, cnt - 1);
+  const int t_lo = (a.window > 0 ? max(0, p_lo - a.window + 1) : 0) >> 4, t_hi = p_hi >> 4;
+  void* const* gkp = a.kspans + (size_t)a.ent_slot[e] * a.span_stride;
+  void* const* gvp = a.vspans + (size_t)a.ent_slot[e] * a.span_stride;
+
+  // this wave's heads for the scores: wave + 8 i
+  u32x4_t qf[HPW][KS];
+  float mul[HPW], mrun[HPW], lrun[HPW];
+#pragma unroll
+  for (int i = 0; i < HPW; ++i) {
+    const int h = wave + 8 * i;
+    mul[i] = a.scale * (a.temp && h < H ? ld_any(a.temp, h, a.wdt) : 1.f);
+    mrun[i] = -1e30f;
+    lrun[i] = PASS == 1 ? 0.f : 1.f;
+    const float* qrow = a.q + (size_t)(row0 + tq) * a.ldq + (size_t)(h < H ? h : 0) * D;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      qf[i][ks] = u32x4_t{0u, 0u, 0u, 0u};
+      const int d0 = ks * 32 + kb * 8;
+      if (d0 < D && h < H) {
+        const f32x4_t lo = *reinterpret_cast<const f32x4_t*>(qrow + d0);
+        const f32x4_t hi = *reinterpret_cast<const f32x4_t*>(qrow + d0 + 4);
+        qf[i][ks] = u32x4_t{pack_bf16x2(lo[0], lo[1]), pack_bf16x2(lo[2], lo[3]), pack_bf16x2(hi[0], hi[1]), pack_bf16x2(hi[2], hi[3])};
+      }
+    }
+    if (PASS == 2 && h < H) {
+      const float* st = a.stats + ((size_t)(row0 + tq) * H + h) * 2;
+      mrun[i] = st[0];
+      lrun[i] = 1.f / st[1];
+    }
+  }
+  const f32x4_t z4 = {0.f, 0.f, 0.f, 0.f};
+  f32x4_t oacc[OPW][DT];
+#pragma unroll
+  for (int i = 0; i < OPW; ++i)
+#pragma unroll
+    for (int t = 0; t < DT; ++t) oacc[i][t] = z4;
+
+  const int uk = D >> 3, uv = DV >> 3;                         // 16-byte units per key row
+  for (int tile = t_lo; tile <= t_hi; ++tile) {
+    const int key0 = tile * 16, sp = key0 / a.span_len, in = key0 - sp * a.span_len;
+    const int live = min(16, p_hi - key0 + 1);                 // keys of the tile that exist (later ones were never written)
+    const char* kbp = (const char*)gkp[sp] + (size_t)in * G * D * 2;
+    for (int u = tid; u < 16 * G * uk; u += 512) {             // page rows are [key][G][D]
+      const int kin = u / (G * uk), rest = u - kin * (G * uk), g = rest / uk, c8 = rest - g * uk;
+      u32x4_t v = {0u, 0u, 0u, 0u};
+      if (kin < live) v = gload<u32x4_t>(kbp + ((size_t)(kin * G + g) * D + c8 * 8) * 2);
+      *reinterpret_cast<u32x4_t*>(ksm + (g * 16 + kin) * pitchk + c8 * 16) = v;
+    }
+    if (PASS == 2) {
+      const char* vbp = (const char*)gvp[sp] + (size_t)in * G * DV * 2;
+      for (int u = tid; u < 16 * G * uv; u += 512) {
+        const int kin = u / (G * uv), rest = u - kin * (G * uv), g = rest / uv, c8 = rest - g * uv;
+        u32x4_t v = {0u, 0u, 0u, 0u};
+        if (kin < live) v = gload<u32x4_t>(vbp + ((size_t)(kin * G + g) * DV + c8 * 8) * 2);
+        *reinterpret_cast<u32x4_t*>(vsm + (g * 16 + kin) * pitchv + c8 * 16) = v;
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < HPW; ++i) {
+      const int h = wave + 8 * i;
+      if (h < H) {
+        const unsigned char* kt = ksm + ((h / hpg) * 16 + ni) * pitchk + kb * 16;
+        f32x4_t sacc = z4;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+          if (ks * 32 < D) sacc = mfma_bf16t(*reinterpret_cast<const u32x4_t*>(kt + ks * 64), qf[i][ks], sacc);
+        float sv[4], mx = -INFINITY;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int key = key0 + kb * 4 + r;
+          const bool seen = key <= p && (a.window <= 0 || p - key < a.window);
+          sv[r] = seen ? sacc[r] * mul[i] : -INFINITY;
+          mx = fmaxf(mx, sv[r]);
+        }
+        if (PASS == 1) {
+          mx = rows_max(mx);
+          const float mn = fmaxf(mrun[i], mx);
+          float ps = 0.f;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) ps += __expf(sv[r] - mn);
+          lrun[i] = lrun[i] * __expf(mrun[i] - mn) + rows_sum(ps);
+          mrun[i] = mn;
+        } else {
+          const f32x4_t pv = {__expf(sv[0] - mrun[i]) * lrun[i], __expf(sv[1] - mrun[i]) * lrun[i], __expf(sv[2] - mrun[i]) * lrun[i],
+                              __expf(sv[3] - mrun[i]) * lrun[i]};
+          *reinterpret_cast<f32x4_t*>(psm + ((size_t)h * 16 + ni) * 16 + kb * 4) = pv;
+        }
+      }
+    }
+    if (PASS == 2) {
+      __syncthreads();
+      f32x4_t pm[OPW];
+      int oh[OPW];
+#pragma unroll
+      for (int i = 0; i < OPW; ++i) { pm[i] = z4; oh[i] = (blockIdx.z * OPW + i) * 8 + wave; }
+      if (oh[0] < H) {
+        const float* pl = psm + ni * 16 + kb * 4;
+        for (int g = 0; g < H; ++g) {
+          const f32x4_t pv = *reinterpret_cast<const f32x4_t*>(pl + g * 256);
+#pragma unroll
+          for (int i = 0; i < OPW; ++i) {
+            const float tw = oh[i] < H ? ((talk_uniform_ptr)(a.talk32))[oh[i] * H + g] : 0.f;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) pm[i][r] = __builtin_fmaf(tw, pv[r], pm[i][r]);
+          }
+        }
+#pragma unroll
+        for (int i = 0; i < OPW; ++i) {
+          if (oh[i] < H) {
+            const u32x2_t pf = {pack_bf16x2(pm[i][0], pm[i][1]), pack_bf16x2(pm[i][2], pm[i][3])};
+            const unsigned char* tr0 = vsm + ((oh[i] / hpg) * 16 + kb * 4 + (ni >> 2)) * pitchv + (ni & 3) * 8;
+#pragma unroll
+            for (int t = 0; t < DT; ++t)
+              if (t * 16 < DV) oacc[i][t] = mfma_bf16k16(lds_read_tr16(tr0 + t * 32), pf, oacc[i][t]);
+          }
+        }
+      }
+    }
+    __syncthreads();
+  }
+  asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");
+  if (!row_ok) return;
+  if (PASS == 1) {
+    if (kb == 0 && blockIdx.z == 0) {
+#pragma unroll
+      for (int i = 0; i < HPW; ++i) {
+        const int h = wave + 8 * i;
+        if (h < H) {
+          float* st = a.stats + ((size_t)(row0 + tq) * H + h) * 2;
+          st[0] = mrun[i];
+          st[1] = lrun[i];
+        }
+      }
+    }
+    return;
+  }
+#pragma unroll
+  for (int i = 0; i < OPW; ++i) {
+    const int h = (blockIdx.z * OPW + i) * 8 + wave;
+    if (h >= H) continue;
+#pragma unroll
+    for (int t = 0; t < DT; ++t) {
+      if (t * 16 >= DV) continue;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const size_t c = (size_t)h * DV + t * 16 + kb * 4 + r;
+        const float v = oacc[i][t][r];
+        st_any(a.out, (size_t)(row0 + tq) * a.ldo + c, a.odt, a.gate ? v * a.gate[(size_t)(row0 + tq) * a.ldg + c] : v);
+      }
+    }
+  }
+}
+
 }  // namespace
 }  // namespace dihip
 
@@ -244,6 +447,65 @@ int dihip_talk_attn(void* stream, void* out, int out_dtype, long ldo, const floa
     by_h(std::integral_constant<int, DIHIP_BF16>{});
   }
   if (nsplit > 1) hipLaunchKernelGGL(talk_merge_kernel, dim3(T, T >= 256 ? 1 : (H * DV + 1023) / 1024), dim3(256), 0, s, a);
+  return launch_status();
+}
+
+static size_t talk_mc_lds_bytes(int pass, int H, int G, int D, int DV) {
+  size_t b = (size_t)G * 16 * (D + 8) * 2;
+  if (pass == 2) b += (size_t)G * 16 * (DV + 8) * 2 + (size_t)H * 256 * sizeof(float);
+  return b;
+}
+
+/* 1 when the matrix-core form serves these sizes on this device (bf16 pages) */
+int dihip_talk_attn_mc_supported(int H, int G, int D, int DV, int span_len, int cache_dtype) {
+  if (cache_dtype != DIHIP_BF16 || H < 1 || H > 32 || G < 1 || H % G || D % 32 || D > 128 || DV % 16 || DV > 128 || span_len % 16) return 0;
+  return talk_mc_lds_bytes(2, H, G, D, DV) <= 160 * 1024 - 1024;
+}
+
+size_t dihip_talk_attn_mc_workspace_bytes(int T, int H) { return (size_t)T * H * 2 * sizeof(float); }
+
+int dihip_talk_attn_mc(void* stream, void* out, int out_dtype, long ldo, const float* q, long ldq, void* const* kspans, void* const* vspans,
+                       int span_stride, int span_len, const void* temp, int w_dtype, const float* talk32, const float* gate, long ldg,
+                       const int32_t* tok_pos, const int32_t* ent_slot, const int32_t* ent_row0, const int32_t* ent_count, int E, int max_count,
+                       int T, int H, int G, int D, int DV, float scale, int window, void* ws, size_t ws_bytes) {
+  DIHIP_REQUIRE(T >= 0 && E >= 0 && max_count >= 0 && out && q && kspans && vspans && talk32 && tok_pos && ent_slot && ent_row0 && ent_count &&
+                    span_stride > 0 && span_len > 0 && ldo >= (long)H * DV && ldq >= (long)H * D && (!gate || ldg >= (long)H * DV) &&
+                    seq_dtype_ok(out_dtype) && seq_dtype_ok(w_dtype) && E <= 65535, DIHIP_PARAM_ERROR, "talk_attn_mc: bad argument");
+  DIHIP_REQUIRE(dihip_talk_attn_mc_supported(H, G, D, DV, span_len, DIHIP_BF16), DIHIP_EXCEED_LIMIT_ERROR,
+                "talk_attn_mc: sizes the matrix-core form does not serve (H <= 32, D %% 32 == 0 <= 128, DV %% 16 == 0 <= 128)");
+  DIHIP_REQUIRE((ldq & 3) == 0 && (reinterpret_cast<uintptr_t>(q) & 15u) == 0, DIHIP_PARAM_ERROR, "talk_attn_mc: query rows must be 16-byte aligned");
+  DIHIP_REQUIRE(ws && ws_bytes >= dihip_talk_attn_mc_workspace_bytes(T, H) && (reinterpret_cast<uintptr_t>(ws) & 3u) == 0, DIHIP_PARAM_ERROR,
+                "talk_attn_mc: workspace too small");
+  if (T == 0 || E == 0 || max_count == 0) return DIHIP_SUCCESS;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  TalkMcArgs a{out, out_dtype, ldo, q, ldq, kspans, vspans, span_stride, span_len, temp, w_dtype, talk32, gate, ldg, tok_pos, ent_slot, ent_row0,
+               ent_count, H, G, D, DV, scale, window, (float*)ws};
+  const int tiles = (max_count + 15) / 16;
+  const size_t lds1 = talk_mc_lds_bytes(1, H, G, D, DV), lds2 = talk_mc_lds_bytes(2, H, G, D, DV);
+  int status = DIHIP_SUCCESS;
+  auto go = [&](auto hpw, auto opw, auto dmax, auto vmax) {
+    constexpr int HPW = decltype(hpw)::value, OPW = decltype(opw)::value, DMAX = decltype(dmax)::value, VMAX = decltype(vmax)::value;
+    auto k1 = talk_attn_mc_kernel<1, HPW, 1, DMAX, 16>;
+    auto k2 = talk_attn_mc_kernel<2, HPW, OPW, DMAX, VMAX>;
+    if (lds1 > 64 * 1024 && hipFuncSetAttribute(reinterpret_cast<const void*>(k1), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds1) != hipSuccess) status = DIHIP_RUNTIME_ERROR;
+    if (lds2 > 64 * 1024 && hipFuncSetAttribute(reinterpret_cast<const void*>(k2), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds2) != hipSuccess) status = DIHIP_RUNTIME_ERROR;
+    if (status != DIHIP_SUCCESS) { (void)hipGetLastError(); return; }
+    hipLaunchKernelGGL(k1, dim3(tiles, E, 1), dim3(512), lds1, s, a);
+    hipLaunchKernelGGL(k2, dim3(tiles, E, HPW / OPW), dim3(512), lds2, s, a);
+  };
+  auto by_size = [&](auto hpw, auto opw) {
+    using d64 = std::integral_constant<int, 64>;
+    using d128 = std::integral_constant<int, 128>;
+    if (D <= 64) { if (DV <= 64) go(hpw, opw, d64{}, d64{}); else go(hpw, opw, d64{}, d128{}); }
+    else { if (DV <= 64) go(hpw, opw, d128{}, d64{}); else go(hpw, opw, d128{}, d128{}); }
+  };
+  using c1 = std::integral_constant<int, 1>;
+  using c2 = std::integral_constant<int, 2>;
+  using c4 = std::integral_constant<int, 4>;
+  if (H <= 8) by_size(c1{}, c1{});
+  else if (H <= 16) by_size(c2{}, c2{});
+  else by_size(c4{}, c2{});
+  DIHIP_REQUIRE(status == DIHIP_SUCCESS, DIHIP_RUNTIME_ERROR, "talk_attn_mc: the device refused %zu bytes of LDS for a workgroup", lds2);
   return launch_status();
 }
 

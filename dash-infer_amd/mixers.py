@@ -260,6 +260,10 @@ class GroupedQueryAttention:
         self.vtables = [state.add_span_cache(n + ".v", self.G * vdim, cache_dtype) for n in names]
         self.ktable, self.vtable = self.ktables[0], self.vtables[0]
         self.mc = so.gqa_attn_mc_supported(dim, vdim, self.ktable) and self.n_in % 4 == 0 and (heads * dim) % 4 == 0
+        self.talk32, self.talk_mc = None, False
+        if self.talk is not None:
+            self.talk32 = self.talk.float().contiguous()
+            self.talk_mc = so.talk_attn_mc_supported(self.H, self.G, dim, vdim, self.ktable) and self.n_in % 4 == 0
 
     def __call__(self, ctx, h, h16=None, run=0):
         H, G, D, V = self.H, self.G, self.D, self.V
@@ -277,6 +281,11 @@ class GroupedQueryAttention:
         so.qkv_prep_append(a, 0, self.k_lo, self.v_lo, H, G, D, V, self.q_norm, self.k_norm, ctx.eps, self.freq, self.rot_dims, self.layout,
                            self.mag, lam, vin, vout, ktable, vtable, ctx.tok_slot, ctx.tok_pos, maps=self.maps)
         gate = a[:, self.g_lo:] if self.head_gate else None
+        if self.talk is not None and ctx.math == so.MATH_BF16 and self.talk_mc and ctx.max_count >= so.TALK_MC_MIN_ROWS:
+            o = so.talk_attn_mc(a, ktable, vtable, ctx.tok_pos, ctx.ent_slot, ctx.ent_row0, ctx.ent_count, ctx.max_count, H, G, D, V, self.scale,
+                                self.talk32, temp=self.head_temp, gate=a[:, self.g_lo:] if self.elem_gate else None, window=self.window,
+                                out=ctx.act_buffer(H * V))
+            return so.linear(o, self.o, self.o_b, math=ctx.math)
         if self.talk is not None:
             o = so.talk_attn(a, ktable, vtable, ctx.tok_slot, ctx.tok_pos, ctx.max_pos, H, G, D, V, self.scale, self.talk, temp=self.head_temp,
                              gate=a[:, self.g_lo:] if self.elem_gate else None, window=self.window, out=ctx.act_buffer(H * V))

@@ -451,3 +451,24 @@ def talk_attn(q, ktable, vtable, tok_slot, tok_pos, max_pos, H, G, D, DV, scale,
                                 _rows(gate) if gate is not None else 0, ptr(tok_slot), ptr(tok_pos), T, H, G, D, DV, float(scale), window,
                                 int(nsplit), ptr(ws), ws.numel()), "dihip_talk_attn")
     return o
+
+
+TALK_MC_MIN_ROWS = 16    # steps whose largest portion has fewer rows (decoding) take the split row kernel
+
+
+def talk_attn_mc_supported(H, G, D, DV, table):
+    return bool(lib().dihip_talk_attn_mc_supported(int(H), int(G), int(D), int(DV), table.span_len, _DT[table.dtype]))
+
+
+def talk_attn_mc(q, ktable, vtable, tok_pos, ent_slot, ent_row0, ent_count, max_count, H, G, D, DV, scale, talk32, temp=None, gate=None, window=0,
+                 out=None):
+    """the matrix-core form of talk_attn (bf16 pages): rows as portions; talk32: the mixing matrix as f32 [H, H]"""
+    T, E = q.shape[0], ent_slot.shape[0]
+    o = out if out is not None else torch.empty(T, H * DV, dtype=torch.float32, device=q.device)
+    ws = torch.empty(int(lib().dihip_talk_attn_mc_workspace_bytes(T, H)), dtype=torch.uint8, device=q.device)
+    assert talk32.dtype == torch.float32 and talk32.shape == (H, H) and talk32.is_contiguous() and q.dtype == torch.float32
+    check(lib().dihip_talk_attn_mc(stream(), ptr(o), dt(o), _rows(o), ptr(q), _rows(q), ptr(ktable.ptrs), ptr(vtable.ptrs), ktable.max_spans,
+                                   ktable.span_len, ptr(temp), dt(temp) if temp is not None else F32_CODE, ptr(talk32), ptr(gate),
+                                   _rows(gate) if gate is not None else 0, ptr(tok_pos), ptr(ent_slot), ptr(ent_row0), ptr(ent_count), E,
+                                   int(max_count), T, H, G, D, DV, float(scale), int(window or 0), ptr(ws), ws.numel()), "dihip_talk_attn_mc")
+    return o

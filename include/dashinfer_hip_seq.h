@@ -104,6 +104,18 @@ int dihip_talk_attn(void* stream, void* out, int out_dtype, long ldo, const floa
                     long ldg, const int32_t* tok_slot, const int32_t* tok_pos, int T, int H, int G, int D, int DV, float scale,
                     int window, int nsplit, void* ws, size_t ws_bytes);
 
+/* The same attention on the matrix cores (bf16 pages; H <= 32, D % 32 == 0 <= 128, DV % 16 == 0 <= 128, span_len % 16 == 0): rows as
+ * portions (ent_slot / ent_row0 / ent_count [E], max_count = the largest portion: a host number that sizes the grid), the whole key
+ * walk of a 16-row tile in one workgroup.  talk32: the mixing matrix as f32 [H, H].  The weights are mixed in f32 and handed to the
+ * value product in bf16.  Workspace: the (maximum, denominator) of every (row, head). */
+int dihip_talk_attn_mc_supported(int H, int G, int D, int DV, int span_len, int cache_dtype);
+size_t dihip_talk_attn_mc_workspace_bytes(int T, int H);
+int dihip_talk_attn_mc(void* stream, void* out, int out_dtype, long ldo, const float* q, long ldq, void* const* kspans,
+                       void* const* vspans, int span_stride, int span_len, const void* temp, int w_dtype, const float* talk32,
+                       const float* gate, long ldg, const int32_t* tok_pos, const int32_t* ent_slot, const int32_t* ent_row0,
+                       const int32_t* ent_count, int E, int max_count, int T, int H, int G, int D, int DV, float scale, int window,
+                       void* ws, size_t ws_bytes);
+
 /* Grouped-query attention, step 1: per token the rows qkv[t] hold q [H, maps, D] at column q_off, k [G, maps, D] at k_off,
  * v [G, DV] at v_off (f32; maps = the softmax maps per head, 1 for ordinary attention).  Every query and key head is divided by its root mean square and scaled by qnorm / knorm [D] (NULL: no norm),
  * then rotated on its first rot_dims dimensions by the angles tok_pos[t] * freq[i] (f32 product; layout 0: dimension 2i

@@ -188,6 +188,10 @@ TALK_SHAPES = {
     "as_many_kv_heads": dict(heads=4, kv_heads=4, dim=32, vdim=64, rot_dims=16, window=64),
     "one_key": dict(heads=2, kv_heads=2, dim=8, vdim=200, rot_dims=0, window=1),
     "never_binds": dict(heads=16, kv_heads=4, dim=8, vdim=8, rot_dims=4, window=1000, base=77.0),
+    # sizes of the matrix-core form: two and four heads per wave, output heads shared between two workgroups, heads past a multiple of 8
+    "tiles_16_heads": dict(heads=16, kv_heads=2, dim=64, vdim=32, rot_dims=32, window=50),
+    "tiles_32_heads": dict(heads=32, kv_heads=8, dim=32, vdim=16, rot_dims=32, window=33),
+    "tiles_12_heads": dict(heads=12, kv_heads=3, dim=96, vdim=80, rot_dims=48, window=129),
 }
 
 
