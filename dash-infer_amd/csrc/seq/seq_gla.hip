@@ -237,6 +237,10 @@ using namespace dihip;
 
 extern "C" {
 
+// columns per thread: two where the registers allow (D <= 128) and the head has more than 64 value columns -- and for 64 < D <= 128
+// also where it has not: the one-column form of that size needs more registers than a lane has (it ran from scratch memory, ten
+// times slower); the second column of such a thread is past the head and idle
+static int gla_cpt(int D, int DV) { return D <= 128 && (DV > 64 || D > 64) ? 2 : 1; }
 static int gla_dpad(int D) { return D <= 64 ? 64 : (D <= 128 ? 128 : 256); }
 
 // the state kernels over records that a rows kernel has written
@@ -276,7 +280,7 @@ int dihip_gla(void* stream, float* out, long ldo, const float* q, long ldq, cons
                     ent_count && ldo >= (long)H * DV && ldq >= (long)H * D && ldk >= (long)H * D && ldz >= (long)H * D && ldv >= (long)H * DV &&
                     tau > 0.f, DIHIP_PARAM_ERROR, "gla: bad argument");
   DIHIP_REQUIRE(D <= 256, DIHIP_EXCEED_LIMIT_ERROR, "gla: more than 256 key channels per head (%d)", D);
-  const int cpt = (DV > 64 && D <= 128) ? 2 : 1;   // columns per thread: two where the registers allow
+  const int cpt = gla_cpt(D, DV);
   const int cbs = (DV + 64 * cpt - 1) / (64 * cpt);
   DIHIP_REQUIRE((long)H * cbs <= 65535 && E <= 65535, DIHIP_PARAM_ERROR, "gla: too many heads or portions for one launch");
   DIHIP_REQUIRE(ws && ws_bytes >= dihip_gla_workspace_bytes(T, E, max_count, H, D, DV, chunked) && (reinterpret_cast<uintptr_t>(ws) & 3u) == 0,
@@ -300,7 +304,7 @@ int dihip_ssd(void* stream, float* out, long ldo, const float* x, long ldx, cons
                     a_log && state && ent_slot && ent_row0 && ent_count && ldo >= (long)H * DV && ldx >= (long)H * DV && ldb >= (long)G * D &&
                     ldc >= (long)G * D && lddt >= H && seq_dtype_ok(w_dtype), DIHIP_PARAM_ERROR, "ssd: bad argument");
   DIHIP_REQUIRE(D <= 256, DIHIP_EXCEED_LIMIT_ERROR, "ssd: more than 256 state channels per head (%d)", D);
-  const int cpt = (DV > 64 && D <= 128) ? 2 : 1;
+  const int cpt = gla_cpt(D, DV);
   const int cbs = (DV + 64 * cpt - 1) / (64 * cpt);
   DIHIP_REQUIRE((long)H * cbs <= 65535 && E <= 65535, DIHIP_PARAM_ERROR, "ssd: too many heads or portions for one launch");
   DIHIP_REQUIRE(ws && ws_bytes >= dihip_gla_workspace_bytes(T, E, max_count, H, D, DV, chunked) && (reinterpret_cast<uintptr_t>(ws) & 3u) == 0,

@@ -43,6 +43,7 @@ __device__ __forceinline__ float talk_score(const TalkArgs& a, const float* __re
   const char* kr = (const char*)ktab[j / a.span_len] + ((size_t)(j % a.span_len) * a.G + g) * a.D * ES;
   float d = 0.f;
   if ((a.D & 7) == 0) {
+#pragma unroll 4
     for (int r = 0; r < a.D; r += 8) {
       float kv[8];
       if (CT == DIHIP_F32) {
@@ -99,6 +100,7 @@ __global__ __launch_bounds__(256) void talk_apply_kernel(TalkArgs a) {
   __shared__ float ps[TALK_MAX_H][64];
   __shared__ float pw[4][64];
   __shared__ float mx_s[TALK_MAX_H], inv_s[TALK_MAX_H];
+  __shared__ const char* vrow_s[64];
   const int t = blockIdx.x, s = blockIdx.y, lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int H = a.H, DV = a.DV, hpg = H / a.G;
@@ -129,6 +131,10 @@ __global__ __launch_bounds__(256) void talk_apply_kernel(TalkArgs a) {
   __syncthreads();
   for (int j0 = lo; j0 < hi; j0 += 64) {
     const int j = j0 + lane, cnt = min(64, hi - j0);
+    if (threadIdx.x < 64) {                            // the chunk's value rows (key/value head 0), published by the barrier below
+      const int jk = j0 + threadIdx.x;
+      vrow_s[threadIdx.x] = jk < hi ? (const char*)vtab[jk / a.span_len] + (size_t)(jk % a.span_len) * a.G * DV * ES : nullptr;
+    }
 #pragma unroll
     for (int i = 0; i < HPW; ++i) {
       const int h = i * 4 + wave;
@@ -151,16 +157,26 @@ __global__ __launch_bounds__(256) void talk_apply_kernel(TalkArgs a) {
       pw[wave][lane] = pm;
       __syncthreads();
       if (h < H) {
-        const int gv = h / hpg;
-        for (int jj = 0; jj < cnt; ++jj) {
-          const int jk = j0 + jj;
-          const char* vr = (const char*)vtab[jk / a.span_len] + ((size_t)(jk % a.span_len) * a.G + gv) * DV * ES;
-          const float pj = pw[wave][jj];
+        const size_t voff = (size_t)(h / hpg) * DV * ES;
+        for (int jj = 0; jj < cnt; jj += 8) {        // eight keys' loads in flight; the sums run in key order
+          float pj[8], vv[8][RV];
 #pragma unroll
-          for (int v = 0; v < RV; ++v) {
-            const int r = v * 64 + lane;
-            if (r < DV) acc[i][v] = __builtin_fmaf(pj, load_ft<CT>(vr, r), acc[i][v]);
+          for (int x = 0; x < 8; ++x) {
+            const bool in = jj + x < cnt;
+            const char* vr = in ? vrow_s[jj + x] + voff : nullptr;
+            pj[x] = in ? pw[wave][jj + x] : 0.f;
+#pragma unroll
+            for (int v = 0; v < RV; ++v) {
+              const int r = v * 64 + lane;
+              vv[x][v] = in && r < DV ? load_ft<CT>(vr, r) : 0.f;
+            }
           }
+#pragma unroll
+          for (int x = 0; x < 8; ++x)
+            if (jj + x < cnt) {
+#pragma unroll
+              for (int v = 0; v < RV; ++v) acc[i][v] = __builtin_fmaf(pj[x], vv[x][v], acc[i][v]);
+            }
         }
       }
       __syncthreads();
@@ -187,6 +203,114 @@ __global__ __launch_bounds__(256) void talk_merge_kernel(TalkArgs a) {
     float v = 0.f;
     for (int s = 0; s < a.nsplit; ++s) v += a.part[((size_t)t * a.nsplit + s) * N + c];
     st_any(a.out, (size_t)t * a.ldo + c, a.odt, a.gate ? v * a.gate[(size_t)t * a.ldg + c] : v);
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ few rows (decoding)
+// With few rows one workgroup per (row, part of the walk) leaves the chip empty and every wave waits on one load after the other.
+// The same two passes spread over the heads:
+//   talk_scores   one wave per (row, head, 64-key chunk of the row's window): the raw scores -> S [row][head][key], the chunk's
+//                 maximum and denominator -> stats
+//   talk_mix      one workgroup per (row, OUTPUT head, 256 keys): all heads' statistics merged (chunks in order), the mixed weight of
+//                 every key from S, then the values of the head's key/value head -- 64 keys per wave, eight loads in flight, the four
+//                 waves' sums added in order
+// and talk_merge adds the parts.
+struct TalkFewArgs {
+  TalkArgs a;
+  float* S; int Wp, nchunk;      // S [T][H][Wp] (Wp = nchunk * 64), stats [T][nchunk][H][2]
+};
+
+template <int CT>
+__global__ __launch_bounds__(64) void talk_scores_kernel(TalkFewArgs f) {
+  const TalkArgs& a = f.a;
+  const int t = blockIdx.x, h = blockIdx.y, c = blockIdx.z, lane = threadIdx.x;
+  const int pos = a.tok_pos[t];
+  const int w_lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
+  const int j = w_lo + c * 64 + lane;
+  const bool valid = j <= pos;
+  void* const* ktab = a.kspans + (size_t)a.tok_slot[t] * a.span_stride;
+  float sc = -INFINITY;
+  if (valid) sc = talk_score<CT>(a, a.q + (size_t)t * a.ldq + (size_t)h * a.D, ktab, j, h / (a.H / a.G), a.temp ? ld_any(a.temp, h, a.wdt) : 1.f);
+  f.S[((size_t)t * a.H + h) * f.Wp + c * 64 + lane] = sc;
+  const float mx = wave_max(sc);
+  const float sum = wave_sum(valid ? expf(sc - mx) : 0.f);
+  if (lane == 0) {
+    float* st = a.stats + (((size_t)t * f.nchunk + c) * a.H + h) * 2;
+    st[0] = mx;
+    st[1] = sum;
+  }
+}
+
+template <int CT, int RV>
+__global__ __launch_bounds__(256) void talk_mix_kernel(TalkFewArgs f) {
+  const TalkArgs& a = f.a;
+  __shared__ float mx_s[TALK_MAX_H], inv_s[TALK_MAX_H];
+  __shared__ float pm_s[256];
+  __shared__ const char* vrow_s[256];
+  __shared__ float red_s[4][64 * RV];
+  const int t = blockIdx.x, h = blockIdx.y, part = blockIdx.z, tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int H = a.H, DV = a.DV;
+  const int pos = a.tok_pos[t];
+  const int w_lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
+  const int nch = (pos - w_lo) / 64 + 1;                       // chunks of this row
+  for (int g = tid; g < H; g += 256) {
+    const float* st = a.stats + ((size_t)t * f.nchunk * H + g) * 2;
+    float mx = -INFINITY;
+    for (int c = 0; c < nch; ++c) mx = fmaxf(mx, st[(size_t)c * H * 2]);
+    float den = 0.f;
+    for (int c = 0; c < nch; ++c) {
+      const float m = st[(size_t)c * H * 2];
+      if (m != -INFINITY) den += st[(size_t)c * H * 2 + 1] * expf(m - mx);
+    }
+    mx_s[g] = mx;
+    inv_s[g] = 1.f / den;
+  }
+  __syncthreads();
+  constexpr size_t ES = CT == DIHIP_F32 ? 4 : 2;
+  const int k = part * 256 + tid, j = w_lo + k;                // this thread's key, counted from the window's start
+  const bool valid = j <= pos;
+  float pm = 0.f;
+  if (valid) {
+    const float* srow = f.S + (size_t)t * H * f.Wp + k;
+    for (int g = 0; g < H; ++g) pm = __builtin_fmaf(ld_any(a.talk, (size_t)h * H + g, a.wdt), expf(srow[(size_t)g * f.Wp] - mx_s[g]) * inv_s[g], pm);
+  }
+  pm_s[tid] = pm;
+  void* const* vtab = a.vspans + (size_t)a.tok_slot[t] * a.span_stride;
+  vrow_s[tid] = valid ? (const char*)vtab[j / a.span_len] + ((size_t)(j % a.span_len) * a.G + h / (H / a.G)) * DV * ES : nullptr;
+  __syncthreads();
+  float acc[RV];
+#pragma unroll
+  for (int v = 0; v < RV; ++v) acc[v] = 0.f;
+  const int cnt = min(64, pos - (w_lo + part * 256 + wave * 64) + 1);      // live keys of this wave's 64 (<= 0: none)
+  for (int jj = 0; jj < cnt; jj += 8) {
+    float pj[8], vv[8][RV];
+#pragma unroll
+    for (int x = 0; x < 8; ++x) {
+      const bool in = jj + x < cnt;
+      const char* vr = in ? vrow_s[wave * 64 + jj + x] : nullptr;
+      pj[x] = in ? pm_s[wave * 64 + jj + x] : 0.f;
+#pragma unroll
+      for (int v = 0; v < RV; ++v) {
+        const int r = v * 64 + lane;
+        vv[x][v] = in && r < DV ? load_ft<CT>(vr, r) : 0.f;
+      }
+    }
+#pragma unroll
+    for (int x = 0; x < 8; ++x)
+      if (jj + x < cnt) {
+#pragma unroll
+        for (int v = 0; v < RV; ++v) acc[v] = __builtin_fmaf(pj[x], vv[x][v], acc[v]);
+      }
+  }
+#pragma unroll
+  for (int v = 0; v < RV; ++v) red_s[wave][v * 64 + lane] = acc[v];
+  __syncthreads();
+  for (int r = tid; r < DV; r += 256) {
+    const float v = ((red_s[0][r] + red_s[1][r]) + red_s[2][r]) + red_s[3][r];
+    const size_t c = (size_t)h * DV + r;
+    if (a.nsplit > 1) a.part[((size_t)t * a.nsplit + part) * H * DV + c] = v;
+    else st_any(a.out, (size_t)t * a.ldo + c, a.odt, a.gate ? v * a.gate[(size_t)t * a.ldg + c] : v);
   }
 }
 
@@ -447,6 +571,46 @@ int dihip_talk_attn(void* stream, void* out, int out_dtype, long ldo, const floa
     by_h(std::integral_constant<int, DIHIP_BF16>{});
   }
   if (nsplit > 1) hipLaunchKernelGGL(talk_merge_kernel, dim3(T, T >= 256 ? 1 : (H * DV + 1023) / 1024), dim3(256), 0, s, a);
+  return launch_status();
+}
+
+/* Few rows (decoding): the same result with the work spread over (row, head, chunk) -- see talk_scores / talk_mix.  max_keys: a host
+ * bound on the keys any row reads (min(window, last position + 1)).  Workspace: scores, statistics and parts. */
+static int talk_few_chunks(int max_keys) { return (max_keys + 63) / 64; }
+size_t dihip_talk_attn_few_workspace_bytes(int T, int H, int DV, int max_keys) {
+  const int nchunk = talk_few_chunks(max_keys), nparts = (nchunk + 3) / 4;
+  return ((size_t)T * H * nchunk * 64 + (size_t)T * nchunk * H * 2 + (nparts > 1 ? (size_t)T * nparts * H * DV : 0)) * sizeof(float);
+}
+
+int dihip_talk_attn_few(void* stream, void* out, int out_dtype, long ldo, const float* q, long ldq, void* const* kspans, void* const* vspans,
+                        int span_stride, int span_len, int cache_dtype, const void* temp, const void* talk, int w_dtype, const float* gate, long ldg,
+                        const int32_t* tok_slot, const int32_t* tok_pos, int T, int H, int G, int D, int DV, float scale, int window, int max_keys,
+                        void* ws, size_t ws_bytes) {
+  DIHIP_REQUIRE(T >= 0 && out && q && kspans && vspans && talk && tok_slot && tok_pos && span_stride > 0 && span_len > 0 && H > 0 && G > 0 &&
+                    H % G == 0 && D > 0 && DV > 0 && ldo >= (long)H * DV && ldq >= (long)H * D && (!gate || ldg >= (long)H * DV) && max_keys >= 1 &&
+                    seq_dtype_ok(out_dtype) && seq_dtype_ok(cache_dtype) && seq_dtype_ok(w_dtype), DIHIP_PARAM_ERROR, "talk_attn_few: bad argument");
+  DIHIP_REQUIRE(H <= TALK_MAX_H && DV <= 256, DIHIP_EXCEED_LIMIT_ERROR, "talk_attn_few: at most %d heads and values of at most 256 elements", TALK_MAX_H);
+  const int nchunk = talk_few_chunks(max_keys), nparts = (nchunk + 3) / 4;
+  DIHIP_REQUIRE(nchunk <= 65535 && H <= 65535, DIHIP_PARAM_ERROR, "talk_attn_few: too many keys for one launch");
+  DIHIP_REQUIRE(ws && ws_bytes >= dihip_talk_attn_few_workspace_bytes(T, H, DV, max_keys) && (reinterpret_cast<uintptr_t>(ws) & 3u) == 0,
+                DIHIP_PARAM_ERROR, "talk_attn_few: workspace too small");
+  if (T == 0) return DIHIP_SUCCESS;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  float* S = (float*)ws;
+  float* stats = S + (size_t)T * H * nchunk * 64;
+  TalkFewArgs f{TalkArgs{out, out_dtype, ldo, q, ldq, kspans, vspans, span_stride, span_len, temp, talk, w_dtype, gate, ldg, tok_slot, tok_pos,
+                         H, G, D, DV, scale, window, nparts, stats, stats + (size_t)T * nchunk * H * 2},
+                S, nchunk * 64, nchunk};
+  auto go = [&](auto ct) {
+    constexpr int CT = decltype(ct)::value;
+    hipLaunchKernelGGL(talk_scores_kernel<CT>, dim3(T, H, nchunk), dim3(64), 0, s, f);
+    if (DV <= 64) hipLaunchKernelGGL((talk_mix_kernel<CT, 1>), dim3(T, H, nparts), dim3(256), 0, s, f);
+    else if (DV <= 128) hipLaunchKernelGGL((talk_mix_kernel<CT, 2>), dim3(T, H, nparts), dim3(256), 0, s, f);
+    else hipLaunchKernelGGL((talk_mix_kernel<CT, 4>), dim3(T, H, nparts), dim3(256), 0, s, f);
+  };
+  if (cache_dtype == DIHIP_F32) go(std::integral_constant<int, DIHIP_F32>{});
+  else go(std::integral_constant<int, DIHIP_BF16>{});
+  if (nparts > 1) hipLaunchKernelGGL(talk_merge_kernel, dim3(T, T >= 256 ? 1 : (H * DV + 1023) / 1024), dim3(256), 0, s, f.a);
   return launch_status();
 }
 

@@ -125,7 +125,12 @@ def operator_table(size, prompt_len):
         a = torch.randn(T, (H + 2 * G) * D + H * V, device=dev) * 0.3
         talk, temp = bf(H, H), bf(H)
         o16 = torch.empty(T, H * V, dtype=torch.bfloat16, device=dev)
-        sec = _time(lambda: so.talk_attn(a, kt, vt, slot, pos, max_pos, H, G, D, V, 0.09, talk, temp=temp, gate=a[:, (H + 2 * G) * D:], window=win, out=o16), 3)
+        gate = a[:, (H + 2 * G) * D:]
+        if T >= so.TALK_MC_MIN_ROWS and so.talk_attn_mc_supported(H, G, D, V, kt):      # as the mixer chooses: matrix cores for portions, the split row kernel for few rows
+            talk32 = talk.float()
+            sec = _time(lambda: so.talk_attn_mc(a, kt, vt, pos, e_slot, e_row0, e_cnt, T, H, G, D, V, 0.09, talk32, temp=temp, gate=gate, window=win, out=o16), 3)
+        else:
+            sec = _time(lambda: so.talk_attn(a, kt, vt, slot, pos, max_pos, H, G, D, V, 0.09, talk, temp=temp, gate=gate, window=win, out=o16), 3)
         keys = sum(min(int(p) + 1, win) for p in pos.tolist())
         fl_mm, fl_mix = 2.0 * keys * H * (2 * D + V), 2.0 * keys * H * H      # two score passes + values on the matrix cores; the mix in f32
         by = 2.0 * G * (D + V) * min(prompt_len, win + T) + 4.0 * T * H * (D + 2 * V)

@@ -62,6 +62,9 @@ _SIGS = {
     "dihip_talk_attn_workspace_bytes": (sz, [i32, i32, i32, i32]),
     "dihip_talk_attn": (i32, [vp, vp, i32, lng, vp, lng, vp, vp, i32, i32, i32, vp, vp, i32, vp, lng, vp, vp, i32, i32, i32, i32, i32, f32, i32, i32,
                               vp, sz]),
+    "dihip_talk_attn_few_workspace_bytes": (sz, [i32, i32, i32, i32]),
+    "dihip_talk_attn_few": (i32, [vp, vp, i32, lng, vp, lng, vp, vp, i32, i32, i32, vp, vp, i32, vp, lng, vp, vp, i32, i32, i32, i32, i32, f32, i32, i32,
+                                  vp, sz]),
     "dihip_talk_attn_mc_supported": (i32, [i32, i32, i32, i32, i32, i32]),
     "dihip_talk_attn_mc_workspace_bytes": (sz, [i32, i32]),
     "dihip_talk_attn_mc": (i32, [vp, vp, i32, lng, vp, lng, vp, vp, i32, i32, vp, i32, vp, vp, lng, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, i32,

@@ -432,6 +432,7 @@ def ssd(x, B, Cq, dtr, dt_bias, a_log, state, ent_slot, ent_row0, ent_count, max
 
 
 TALK_MAX_HEADS = 64
+TALK_FEW_ROWS = 64      # steps of at most this many rows spread the attention with mixed maps over (row, head, chunk) workgroups
 
 
 def talk_attn(q, ktable, vtable, tok_slot, tok_pos, max_pos, H, G, D, DV, scale, talk, temp=None, gate=None, window=0, out=None, nsplit=None):
@@ -441,11 +442,18 @@ def talk_attn(q, ktable, vtable, tok_slot, tok_pos, max_pos, H, G, D, DV, scale,
     T = q.shape[0]
     window = int(window or 0)
     o = out if out is not None else torch.empty(T, H * DV, dtype=torch.float32, device=q.device)
-    if nsplit is None:       # fill the chip: one workgroup per (row, part), at least 128 keys a part
-        keys = min(max_pos + 1, window) if window > 0 else max_pos + 1
-        nsplit = max(1, min(256 // max(T, 1), (keys + 127) // 128))
-    ws = torch.empty(int(lib().dihip_talk_attn_workspace_bytes(T, H, DV, nsplit)), dtype=torch.uint8, device=q.device)
     assert talk.shape == (H, H) and talk.is_contiguous() and (temp is None or (temp.dtype == talk.dtype and temp.shape == (H,)))
+    keys = min(max_pos + 1, window) if window > 0 else max_pos + 1
+    if nsplit is None and T <= TALK_FEW_ROWS:      # few rows (decoding): the work spread over rows, heads and chunks
+        ws = torch.empty(int(lib().dihip_talk_attn_few_workspace_bytes(T, H, DV, keys)), dtype=torch.uint8, device=q.device)
+        check(lib().dihip_talk_attn_few(stream(), ptr(o), dt(o), _rows(o), ptr(q), _rows(q), ptr(ktable.ptrs), ptr(vtable.ptrs), ktable.max_spans,
+                                        ktable.span_len, _DT[ktable.dtype], ptr(temp), ptr(talk), dt(talk), ptr(gate),
+                                        _rows(gate) if gate is not None else 0, ptr(tok_slot), ptr(tok_pos), T, H, G, D, DV, float(scale), window,
+                                        int(keys), ptr(ws), ws.numel()), "dihip_talk_attn_few")
+        return o
+    if nsplit is None:       # one workgroup per (row, part of the walk)
+        nsplit = max(1, min(256 // max(T, 1), (keys + 63) // 64))
+    ws = torch.empty(int(lib().dihip_talk_attn_workspace_bytes(T, H, DV, nsplit)), dtype=torch.uint8, device=q.device)
     check(lib().dihip_talk_attn(stream(), ptr(o), dt(o), _rows(o), ptr(q), _rows(q), ptr(ktable.ptrs), ptr(vtable.ptrs), ktable.max_spans,
                                 ktable.span_len, _DT[ktable.dtype], ptr(temp), ptr(talk), dt(talk), ptr(gate),
                                 _rows(gate) if gate is not None else 0, ptr(tok_slot), ptr(tok_pos), T, H, G, D, DV, float(scale), window,

@@ -104,6 +104,13 @@ int dihip_talk_attn(void* stream, void* out, int out_dtype, long ldo, const floa
                     long ldg, const int32_t* tok_slot, const int32_t* tok_pos, int T, int H, int G, int D, int DV, float scale,
                     int window, int nsplit, void* ws, size_t ws_bytes);
 
+/* The same attention for few rows (decoding): the work spread over (row, head, 64-key chunk) workgroups.  max_keys: a host bound on
+ * the keys a row reads (min(window, last position + 1)).  Workspace: the raw scores, the chunks' statistics and the parts. */
+size_t dihip_talk_attn_few_workspace_bytes(int T, int H, int DV, int max_keys);
+int dihip_talk_attn_few(void* stream, void* out, int out_dtype, long ldo, const float* q, long ldq, void* const* kspans,
+                        void* const* vspans, int span_stride, int span_len, int cache_dtype, const void* temp, const void* talk,
+                        int w_dtype, const float* gate, long ldg, const int32_t* tok_slot, const int32_t* tok_pos, int T, int H, int G,
+                        int D, int DV, float scale, int window, int max_keys, void* ws, size_t ws_bytes);
 /* The same attention on the matrix cores (bf16 pages; H <= 32, D % 32 == 0 <= 128, DV % 16 == 0 <= 128, span_len % 16 == 0): rows as
  * portions (ent_slot / ent_row0 / ent_count [E], max_count = the largest portion: a host number that sizes the grid), the whole key
  * walk of a 16-row tile in one workgroup.  talk32: the mixing matrix as f32 [H, H].  The weights are mixed in f32 and handed to the
