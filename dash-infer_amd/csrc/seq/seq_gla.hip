@@ -52,7 +52,7 @@ __global__ __launch_bounds__(256) void gla_rows_kernel(GlaArgs a) {
 __global__ __launch_bounds__(256) void ssd_rows_kernel(GlaArgs a, const float* __restrict__ dt, long lddt, const void* __restrict__ dt_bias,
                                                        const void* __restrict__ a_log, int wdt, int G) {
   const int t = blockIdx.x, hpg = a.H / G;
-  for (int c = threadIdx.x; c < a.H * a.Dp; c += 256) {
+  for (int c = blockIdx.y * 256 + threadIdx.x; c < a.H * a.Dp; c += 256 * gridDim.y) {     // few rows: a row's records spread over workgroups
     const int h = c / a.Dp, i = c - h * a.Dp;
     float av = 1.f, kv = 0.f, qv = 0.f;
     if (i < a.D) {
@@ -316,7 +316,7 @@ int dihip_ssd(void* stream, float* out, long ldo, const float* x, long ldx, cons
   float* rec = (float*)ws;
   GlaArgs a{out, ldo, Cq, ldc, B, ldb, x, ldx, nullptr, 0, 1.f, 1.f, state, ent_slot, ent_row0, ent_count, H, D, DV, Dp, T,
             rec, rec + (size_t)T * H * 3 * Dp, chunks};
-  hipLaunchKernelGGL(ssd_rows_kernel, dim3(T), dim3(256), 0, s, a, dt, lddt, dt_bias, a_log, w_dtype, G);
+  hipLaunchKernelGGL(ssd_rows_kernel, dim3(T, T >= 64 ? 1 : (H * Dp + 255) / 256), dim3(256), 0, s, a, dt, lddt, dt_bias, a_log, w_dtype, G);
   gla_launch_state(s, a, E, chunked, cpt, cbs);
   return launch_status();
 }

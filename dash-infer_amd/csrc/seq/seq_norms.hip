@@ -109,6 +109,7 @@ __global__ __launch_bounds__(256) void gate_group_rmsnorm_kernel(void* __restric
   __shared__ float red[4];
   const int t = blockIdx.x, c0 = blockIdx.y * part;
   float ss = 0.f;
+#pragma unroll 4
   for (int k = threadIdx.x; k < part; k += 256) {
     const int c = c0 + k;
     float v = o[(size_t)t * ldo + c];
@@ -118,6 +119,7 @@ __global__ __launch_bounds__(256) void gate_group_rmsnorm_kernel(void* __restric
     ss = __builtin_fmaf(v, v, ss);
   }
   const float inv = 1.f / sqrtf(block256_sum(ss, red) / (float)part + eps);
+#pragma unroll 4
   for (int k = threadIdx.x; k < part; k += 256) {     // the same expressions as above: the same bits
     const int c = c0 + k;
     float v = o[(size_t)t * ldo + c];

@@ -257,8 +257,10 @@ __global__ __launch_bounds__(256) void talk_mix_kernel(TalkFewArgs f) {
   for (int g = tid; g < H; g += 256) {
     const float* st = a.stats + ((size_t)t * f.nchunk * H + g) * 2;
     float mx = -INFINITY;
+#pragma unroll 8
     for (int c = 0; c < nch; ++c) mx = fmaxf(mx, st[(size_t)c * H * 2]);
     float den = 0.f;
+#pragma unroll 8
     for (int c = 0; c < nch; ++c) {
       const float m = st[(size_t)c * H * 2];
       if (m != -INFINITY) den += st[(size_t)c * H * 2 + 1] * expf(m - mx);
@@ -273,6 +275,7 @@ __global__ __launch_bounds__(256) void talk_mix_kernel(TalkFewArgs f) {
   float pm = 0.f;
   if (valid) {
     const float* srow = f.S + (size_t)t * H * f.Wp + k;
+#pragma unroll 8
     for (int g = 0; g < H; ++g) pm = __builtin_fmaf(ld_any(a.talk, (size_t)h * H + g, a.wdt), expf(srow[(size_t)g * f.Wp] - mx_s[g]) * inv_s[g], pm);
   }
   pm_s[tid] = pm;
@@ -283,10 +286,10 @@ __global__ __launch_bounds__(256) void talk_mix_kernel(TalkFewArgs f) {
 #pragma unroll
   for (int v = 0; v < RV; ++v) acc[v] = 0.f;
   const int cnt = min(64, pos - (w_lo + part * 256 + wave * 64) + 1);      // live keys of this wave's 64 (<= 0: none)
-  for (int jj = 0; jj < cnt; jj += 8) {
-    float pj[8], vv[8][RV];
+  for (int jj = 0; jj < cnt; jj += 16) {       // sixteen keys' loads in flight; the sums run in key order
+    float pj[16], vv[16][RV];
 #pragma unroll
-    for (int x = 0; x < 8; ++x) {
+    for (int x = 0; x < 16; ++x) {
       const bool in = jj + x < cnt;
       const char* vr = in ? vrow_s[wave * 64 + jj + x] : nullptr;
       pj[x] = in ? pm_s[wave * 64 + jj + x] : 0.f;
@@ -297,7 +300,7 @@ __global__ __launch_bounds__(256) void talk_mix_kernel(TalkFewArgs f) {
       }
     }
 #pragma unroll
-    for (int x = 0; x < 8; ++x)
+    for (int x = 0; x < 16; ++x)
       if (jj + x < cnt) {
 #pragma unroll
         for (int v = 0; v < RV; ++v) acc[v] = __builtin_fmaf(pj[x], vv[x][v], acc[v]);
