@@ -130,6 +130,186 @@ __global__ __launch_bounds__(256) void gate_group_rmsnorm_kernel(void* __restric
   }
 }
 
+// ------------------------------------------------------------------------------------------------ register forms
+// A row (or a part of one) of at most NT * EPT elements is loaded ONCE, every load issued before the first use (indices past the
+// end are clamped, so no load hangs on a condition), and stays in registers through the reductions.  Rows of more than 1024
+// elements take 512 or 1024 threads: with few rows in the step a row's time is the length of one thread's chain of dependent
+// instructions, and a looping thread of 256 walks 16 elements of a 4096-wide row one after the other, twice or three times.  The
+// form is chosen by the row's length alone, so a row's bits do not depend on the batch.
+template <int NW>
+__device__ __forceinline__ float tree_sum(const float* r) {
+  if constexpr (NW == 1) return r[0];
+  else return tree_sum<NW / 2>(r) + tree_sum<NW / 2>(r + NW / 2);
+}
+// sum over the NT threads of a block, the same value in every thread; red = NT / 64 floats of LDS; one fixed tree
+template <int NT>
+__device__ __forceinline__ float block_sum(float v, float* red) {
+  v = wave_sum(v);
+  __syncthreads();  // red may still be read from the call before
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  return tree_sum<NT / 64>(red);
+}
+
+template <int WT, int NT, int EPT>
+__global__ __launch_bounds__(NT) void residual_layernorm_reg_kernel(float* x_out, const float* x_in, const float* __restrict__ a, long lda,
+                                                                    const float* __restrict__ b, long ldb, float mult,
+                                                                    const int32_t* __restrict__ row_idx, const void* __restrict__ w,
+                                                                    const void* __restrict__ bias, float eps, void* __restrict__ h, int hdt,
+                                                                    long ldh, int K) {
+  __shared__ float red[NT / 64];
+  const int i = blockIdx.x, tid = threadIdx.x;
+  const size_t r = row_idx ? (size_t)row_idx[i] : (size_t)i;
+  float v[EPT];
+#pragma unroll
+  for (int e = 0; e < EPT; ++e) v[e] = x_in[r * K + min(tid + e * NT, K - 1)];
+  if (a) {
+    float s[EPT];
+#pragma unroll
+    for (int e = 0; e < EPT; ++e) s[e] = a[r * lda + min(tid + e * NT, K - 1)];
+    if (b) {
+#pragma unroll
+      for (int e = 0; e < EPT; ++e) s[e] += b[r * ldb + min(tid + e * NT, K - 1)];
+    }
+#pragma unroll
+    for (int e = 0; e < EPT; ++e) v[e] = __builtin_fmaf(mult, s[e], v[e]);
+  }
+  float sum = 0.f;
+#pragma unroll
+  for (int e = 0; e < EPT; ++e) {
+    const int k = tid + e * NT;
+    if (k < K) {
+      if (x_out) x_out[r * K + k] = v[e];
+      sum += v[e];
+    }
+  }
+  if (!w) return;
+  float g[EPT];
+#pragma unroll
+  for (int e = 0; e < EPT; ++e) g[e] = load_ft<WT>(w, min(tid + e * NT, K - 1));
+  const float mean = block_sum<NT>(sum, red) / (float)K;
+  float ss = 0.f;
+#pragma unroll
+  for (int e = 0; e < EPT; ++e) {
+    const float d = v[e] - mean;
+    if (tid + e * NT < K) ss = __builtin_fmaf(d, d, ss);
+  }
+  const float inv = 1.f / sqrtf(block_sum<NT>(ss, red) / (float)K + eps);
+#pragma unroll
+  for (int e = 0; e < EPT; ++e) {
+    const int k = tid + e * NT;
+    if (k < K) {
+      float y = (v[e] - mean) * inv * g[e];
+      if (bias) y += load_ft<WT>(bias, k);
+      st_any(h, (size_t)i * ldh + k, hdt, y);
+    }
+  }
+}
+
+template <int WT, int NT, int EPT>
+__global__ __launch_bounds__(NT) void polynorm_reg_kernel(void* __restrict__ y, int ydt, long ldy, const float* __restrict__ z, long ldz,
+                                                          const void* __restrict__ coef, float eps, int F) {
+  __shared__ float red[NT / 64];
+  const int t = blockIdx.x, tid = threadIdx.x;
+  const float* zr = z + (size_t)t * ldz;
+  float v[EPT];
+#pragma unroll
+  for (int e = 0; e < EPT; ++e) v[e] = zr[min(tid + e * NT, F - 1)];
+  float s1 = 0.f, s2 = 0.f, s3 = 0.f;
+#pragma unroll
+  for (int e = 0; e < EPT; ++e)
+    if (tid + e * NT < F) {
+      const float v2 = v[e] * v[e], v3 = v2 * v[e];
+      s1 = __builtin_fmaf(v[e], v[e], s1);
+      s2 = __builtin_fmaf(v2, v2, s2);
+      s3 = __builtin_fmaf(v3, v3, s3);
+    }
+  const float c0 = load_ft<WT>(coef, 0) / sqrtf(block_sum<NT>(s1, red) / (float)F + eps);
+  const float c1 = load_ft<WT>(coef, 1) / sqrtf(block_sum<NT>(s2, red) / (float)F + eps);
+  const float c2 = load_ft<WT>(coef, 2) / sqrtf(block_sum<NT>(s3, red) / (float)F + eps);
+  const float c3 = load_ft<WT>(coef, 3);
+#pragma unroll
+  for (int e = 0; e < EPT; ++e) {
+    const int k = tid + e * NT;
+    if (k < F) {
+      const float v2 = v[e] * v[e];
+      st_any(y, (size_t)t * ldy + k, ydt, c0 * v[e] + c1 * v2 + c2 * (v2 * v[e]) + c3);
+    }
+  }
+}
+
+template <int WT, int NT, int EPT>
+__global__ __launch_bounds__(NT) void rmsnorm_pair_reg_kernel(float* __restrict__ y, long ldy, const float* __restrict__ xa, long lda,
+                                                              const void* __restrict__ wa, const float* __restrict__ xb, long ldb,
+                                                              const void* __restrict__ wb, float coef, float eps, int K) {
+  __shared__ float red[NT / 64];
+  const int t = blockIdx.x, tid = threadIdx.x;
+  float va[EPT], vb[EPT], ga[EPT], gb[EPT];
+#pragma unroll
+  for (int e = 0; e < EPT; ++e) {
+    const int k = min(tid + e * NT, K - 1);
+    va[e] = xa[(size_t)t * lda + k];
+    vb[e] = xb[(size_t)t * ldb + k];
+    ga[e] = load_ft<WT>(wa, k);
+    gb[e] = load_ft<WT>(wb, k);
+  }
+  float sa = 0.f, sb = 0.f;
+#pragma unroll
+  for (int e = 0; e < EPT; ++e)
+    if (tid + e * NT < K) {
+      sa = __builtin_fmaf(va[e], va[e], sa);
+      sb = __builtin_fmaf(vb[e], vb[e], sb);
+    }
+  const float ia = 1.f / sqrtf(block_sum<NT>(sa, red) / (float)K + eps);
+  const float ib = 1.f / sqrtf(block_sum<NT>(sb, red) / (float)K + eps);
+#pragma unroll
+  for (int e = 0; e < EPT; ++e) {
+    const int k = tid + e * NT;
+    if (k < K) y[(size_t)t * ldy + k] = coef * (va[e] * ia * ga[e] + vb[e] * ib * gb[e]);
+  }
+}
+
+// grid (rows, groups): a workgroup owns one part of one row
+template <int WT, int NT, int EPT>
+__global__ __launch_bounds__(NT) void gate_group_rmsnorm_reg_kernel(void* __restrict__ y, int ydt, long ldy, const float* __restrict__ o, long ldo,
+                                                                    const float* __restrict__ x, long ldx, const void* __restrict__ skip,
+                                                                    const float* __restrict__ z, long ldz, const void* __restrict__ w,
+                                                                    float eps, int P, int part) {
+  __shared__ float red[NT / 64];
+  const int t = blockIdx.x, c0 = blockIdx.y * part, tid = threadIdx.x;
+  float v[EPT], g[EPT], wv[EPT];
+#pragma unroll
+  for (int e = 0; e < EPT; ++e) {
+    const int c = c0 + min(tid + e * NT, part - 1);
+    v[e] = o[(size_t)t * ldo + c];
+    g[e] = z[(size_t)t * ldz + c];
+    wv[e] = load_ft<WT>(w, c);
+  }
+  if (skip) {
+    float xs[EPT], sk[EPT];
+#pragma unroll
+    for (int e = 0; e < EPT; ++e) {
+      const int c = c0 + min(tid + e * NT, part - 1);
+      xs[e] = x[(size_t)t * ldx + c];
+      sk[e] = load_ft<WT>(skip, c / P);
+    }
+#pragma unroll
+    for (int e = 0; e < EPT; ++e) v[e] = __builtin_fmaf(sk[e], xs[e], v[e]);
+  }
+  float ss = 0.f;
+#pragma unroll
+  for (int e = 0; e < EPT; ++e) {
+    v[e] *= g[e] / (1.f + expf(-g[e]));
+    if (tid + e * NT < part) ss = __builtin_fmaf(v[e], v[e], ss);
+  }
+  const float inv = 1.f / sqrtf(block_sum<NT>(ss, red) / (float)part + eps);
+#pragma unroll
+  for (int e = 0; e < EPT; ++e) {
+    const int k = tid + e * NT;
+    if (k < part) st_any(y, (size_t)t * ldy + c0 + k, ydt, v[e] * inv * wv[e]);
+  }
+}
+
 // ckv: rows [R latent | rot shared key part]; q_rot: rows [H][rot]; ql: rows [H][Rp], the absorbed queries in the first R columns
 // of every head.  Rotation of the two halves of the rot dimensions: (u, v) -> (u cos - v sin, v cos + u sin), angle = pos * freq[i].
 template <int WT>
@@ -183,6 +363,22 @@ using namespace dihip;
     else hipLaunchKernelGGL(kernel<DIHIP_BF16>, __VA_ARGS__);                \
   } while (0)
 
+// the register form of `kernel` that holds n elements per workgroup, or the looping form (256 threads) beyond 16384
+#define BY_WT_ROW(kernel, n, wdt, grid, stream, ...)                                                                     \
+  do {                                                                                                                   \
+    if ((n) <= 1024) BY_WT_REG(kernel##_reg_kernel, 256, 4, wdt, grid, stream, __VA_ARGS__);                             \
+    else if ((n) <= 2048) BY_WT_REG(kernel##_reg_kernel, 512, 4, wdt, grid, stream, __VA_ARGS__);                        \
+    else if ((n) <= 4096) BY_WT_REG(kernel##_reg_kernel, 1024, 4, wdt, grid, stream, __VA_ARGS__);                       \
+    else if ((n) <= 8192) BY_WT_REG(kernel##_reg_kernel, 1024, 8, wdt, grid, stream, __VA_ARGS__);                       \
+    else if ((n) <= 16384) BY_WT_REG(kernel##_reg_kernel, 1024, 16, wdt, grid, stream, __VA_ARGS__);                     \
+    else BY_WT(kernel##_kernel, wdt, grid, dim3(256), 0, stream, __VA_ARGS__);                                           \
+  } while (0)
+#define BY_WT_REG(kernel, NT, EPT, wdt, grid, stream, ...)                                                               \
+  do {                                                                                                                   \
+    if ((wdt) == DIHIP_F32) hipLaunchKernelGGL((kernel<DIHIP_F32, NT, EPT>), grid, dim3(NT), 0, stream, __VA_ARGS__);    \
+    else hipLaunchKernelGGL((kernel<DIHIP_BF16, NT, EPT>), grid, dim3(NT), 0, stream, __VA_ARGS__);                      \
+  } while (0)
+
 extern "C" {
 
 int dihip_residual_layernorm(void* stream, float* x_out, const float* x_in, const float* a, long lda, const float* b, long ldb, float mult,
@@ -191,8 +387,8 @@ int dihip_residual_layernorm(void* stream, float* x_out, const float* x_in, cons
   DIHIP_REQUIRE(M >= 0 && K > 0 && x_in && (!a || lda >= K) && (!b || (a && ldb >= K)) && (!w || (h && ldh >= K)) && (!row_idx || !x_out) &&
                     (x_out || !a) && seq_dtype_ok(w_dtype) && seq_dtype_ok(h_dtype), DIHIP_PARAM_ERROR, "residual_layernorm: bad argument");
   if (M == 0) return DIHIP_SUCCESS;
-  BY_WT(residual_layernorm_kernel, w_dtype, dim3(M), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), x_out, x_in, a, lda, b, ldb, mult,
-        row_idx, w, bias, eps, h, h_dtype, ldh, K);
+  BY_WT_ROW(residual_layernorm, K, w_dtype, dim3(M), reinterpret_cast<hipStream_t>(stream), x_out, x_in, a, lda, b, ldb, mult, row_idx, w, bias,
+            eps, h, h_dtype, ldh, K);
   return launch_status();
 }
 
@@ -201,7 +397,7 @@ int dihip_polynorm(void* stream, void* y, int y_dtype, long ldy, const float* z,
   DIHIP_REQUIRE(T >= 0 && F > 0 && y && z && coef && ldy >= F && ldz >= F && seq_dtype_ok(y_dtype) && seq_dtype_ok(w_dtype), DIHIP_PARAM_ERROR,
                 "polynorm: bad argument");
   if (T == 0) return DIHIP_SUCCESS;
-  BY_WT(polynorm_kernel, w_dtype, dim3(T), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), y, y_dtype, ldy, z, ldz, coef, eps, F);
+  BY_WT_ROW(polynorm, F, w_dtype, dim3(T), reinterpret_cast<hipStream_t>(stream), y, y_dtype, ldy, z, ldz, coef, eps, F);
   return launch_status();
 }
 
@@ -210,7 +406,7 @@ int dihip_rmsnorm_pair(void* stream, float* y, long ldy, const float* xa, long l
   DIHIP_REQUIRE(T >= 0 && K > 0 && y && xa && wa && xb && wb && ldy >= K && lda >= K && ldb >= K && seq_dtype_ok(w_dtype), DIHIP_PARAM_ERROR,
                 "rmsnorm_pair: bad argument");
   if (T == 0) return DIHIP_SUCCESS;
-  BY_WT(rmsnorm_pair_kernel, w_dtype, dim3(T), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), y, ldy, xa, lda, wa, xb, ldb, wb, coef, eps, K);
+  BY_WT_ROW(rmsnorm_pair, K, w_dtype, dim3(T), reinterpret_cast<hipStream_t>(stream), y, ldy, xa, lda, wa, xb, ldb, wb, coef, eps, K);
   return launch_status();
 }
 
@@ -221,8 +417,8 @@ int dihip_gate_group_rmsnorm(void* stream, void* y, int y_dtype, long ldy, const
                     ldy >= inner && ldo >= inner && ldz >= inner && (!skip || ldx >= inner) && seq_dtype_ok(y_dtype) && seq_dtype_ok(w_dtype),
                 DIHIP_PARAM_ERROR, "gate_group_rmsnorm: bad argument (the row must divide into the groups)");
   if (T == 0) return DIHIP_SUCCESS;
-  BY_WT(gate_group_rmsnorm_kernel, w_dtype, dim3(T, groups), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), y, y_dtype, ldy, o, ldo, x, ldx,
-        skip, z, ldz, w, eps, P, (int)(inner / groups));
+  BY_WT_ROW(gate_group_rmsnorm, inner / groups, w_dtype, dim3(T, groups), reinterpret_cast<hipStream_t>(stream), y, y_dtype, ldy, o, ldo, x, ldx,
+            skip, z, ldz, w, eps, P, (int)(inner / groups));
   return launch_status();
 }
 

@@ -244,7 +244,7 @@ __global__ __launch_bounds__(64) void talk_scores_kernel(TalkFewArgs f) {
 template <int CT, int RV>
 __global__ __launch_bounds__(256) void talk_mix_kernel(TalkFewArgs f) {
   const TalkArgs& a = f.a;
-  __shared__ float mx_s[TALK_MAX_H], inv_s[TALK_MAX_H];
+  __shared__ float mx_s[TALK_MAX_H], inv_s[TALK_MAX_H], talk_s[TALK_MAX_H];
   __shared__ float pm_s[256];
   __shared__ const char* vrow_s[256];
   __shared__ float red_s[4][64 * RV];
@@ -254,7 +254,8 @@ __global__ __launch_bounds__(256) void talk_mix_kernel(TalkFewArgs f) {
   const int pos = a.tok_pos[t];
   const int w_lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
   const int nch = (pos - w_lo) / 64 + 1;                       // chunks of this row
-  for (int g = tid; g < H; g += 256) {
+  for (int g = tid; g < H; g += 256) {       // every load unconditional: the loads of a round are in flight together
+    talk_s[g] = ld_any(a.talk, (size_t)h * H + g, a.wdt);
     const float* st = a.stats + ((size_t)t * f.nchunk * H + g) * 2;
     float mx = -INFINITY;
 #pragma unroll 8
@@ -262,8 +263,8 @@ __global__ __launch_bounds__(256) void talk_mix_kernel(TalkFewArgs f) {
     float den = 0.f;
 #pragma unroll 8
     for (int c = 0; c < nch; ++c) {
-      const float m = st[(size_t)c * H * 2];
-      if (m != -INFINITY) den += st[(size_t)c * H * 2 + 1] * expf(m - mx);
+      const float m = st[(size_t)c * H * 2], sm = st[(size_t)c * H * 2 + 1];
+      den += m != -INFINITY ? sm * expf(m - mx) : 0.f;
     }
     mx_s[g] = mx;
     inv_s[g] = 1.f / den;
@@ -276,7 +277,7 @@ __global__ __launch_bounds__(256) void talk_mix_kernel(TalkFewArgs f) {
   if (valid) {
     const float* srow = f.S + (size_t)t * H * f.Wp + k;
 #pragma unroll 8
-    for (int g = 0; g < H; ++g) pm = __builtin_fmaf(ld_any(a.talk, (size_t)h * H + g, a.wdt), expf(srow[(size_t)g * f.Wp] - mx_s[g]) * inv_s[g], pm);
+    for (int g = 0; g < H; ++g) pm = __builtin_fmaf(talk_s[g], expf(srow[(size_t)g * f.Wp] - mx_s[g]) * inv_s[g], pm);
   }
   pm_s[tid] = pm;
   void* const* vtab = a.vspans + (size_t)a.tok_slot[t] * a.span_stride;
@@ -289,22 +290,18 @@ __global__ __launch_bounds__(256) void talk_mix_kernel(TalkFewArgs f) {
   for (int jj = 0; jj < cnt; jj += 16) {       // sixteen keys' loads in flight; the sums run in key order
     float pj[16], vv[16][RV];
 #pragma unroll
-    for (int x = 0; x < 16; ++x) {
-      const bool in = jj + x < cnt;
-      const char* vr = in ? vrow_s[wave * 64 + jj + x] : nullptr;
-      pj[x] = in ? pm_s[wave * 64 + jj + x] : 0.f;
+    for (int x = 0; x < 16; ++x) {             // no load hangs on a condition: past the wave's last live key its row is read again
+      const int kk = wave * 64 + min(jj + x, cnt - 1);      // with weight 0, and lanes past the value's width read its last column
+      const char* vr = vrow_s[kk];
+      pj[x] = jj + x < cnt ? pm_s[kk] : 0.f;
 #pragma unroll
-      for (int v = 0; v < RV; ++v) {
-        const int r = v * 64 + lane;
-        vv[x][v] = in && r < DV ? load_ft<CT>(vr, r) : 0.f;
-      }
+      for (int v = 0; v < RV; ++v) vv[x][v] = load_ft<CT>(vr, min(v * 64 + lane, DV - 1));
     }
 #pragma unroll
-    for (int x = 0; x < 16; ++x)
-      if (jj + x < cnt) {
+    for (int x = 0; x < 16; ++x) {
 #pragma unroll
-        for (int v = 0; v < RV; ++v) acc[v] = __builtin_fmaf(pj[x], vv[x][v], acc[v]);
-      }
+      for (int v = 0; v < RV; ++v) acc[v] = __builtin_fmaf(pj[x], vv[x][v], acc[v]);
+    }
   }
 #pragma unroll
   for (int v = 0; v < RV; ++v) red_s[wave][v * 64 + lane] = acc[v];
