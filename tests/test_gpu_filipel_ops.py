@@ -42,7 +42,8 @@ def rows(rng, n, width, scale=1.0):
 
 
 # ---------------------------------------------------------------------------------------------------------------- row operators
-@pytest.mark.parametrize("K", [50, 72, 1024 + 41])
+# widths of every form of the row kernels: 256, 512 and 1024 threads with 4, 8 and 16 elements each, and the looping form beyond
+@pytest.mark.parametrize("K", [50, 72, 1024 + 41, 3000, 4096 + 8, 9001, 16384 + 40])
 def test_layer_norm_fused_with_the_residual_step(so, K):
     rng = np.random.default_rng(0)
     T = 23
@@ -69,11 +70,12 @@ def test_layer_norm_fused_with_the_residual_step(so, K):
 
 def test_cubic_of_normalised_powers_and_the_dense_feed_forward(so):
     rng = np.random.default_rng(1)
-    z = rng.normal(0, 1.3, (17, 333)).astype(np.float32)
     coef = bf(np.array([0.7, -0.4, 0.25, 0.1]))
-    out = torch.empty(17, 333, device="cuda")
-    so.polynorm(dev(z), dev(coef, torch.bfloat16), 1e-4, out)
-    assert rel_err(out.cpu().numpy(), of.poly_norm(z, coef, 1e-4)) < 3e-6
+    for F in (333, 2500, 8192, 14336 + 3, 17001):
+        z = rng.normal(0, 1.3, (17, F)).astype(np.float32)
+        out = torch.empty(17, F, device="cuda")
+        so.polynorm(dev(z), dev(coef, torch.bfloat16), 1e-4, out)
+        assert rel_err(out.cpu().numpy(), of.poly_norm(z, coef, 1e-4)) < 3e-6, F
     width, ff = 72, 50
     w = of.ff_weights(rng, width, {"kind": "dense", "ff": ff})
     h = rows(rng, 40, width)
@@ -82,13 +84,31 @@ def test_cubic_of_normalised_powers_and_the_dense_feed_forward(so):
         assert rel_err(rig.step([("a", h)])[0], of.dense_ff(h, w, EPS)) < tol
 
 
-def test_two_normed_branches_joined(so):
+@pytest.mark.parametrize("K", [70, 1500, 4100, 8192, 20000])
+def test_two_normed_branches_joined(so, K):
     rng = np.random.default_rng(2)
-    a, b = rng.normal(0, 3.0, (9, 70)).astype(np.float32), rng.normal(0, 0.1, (9, 70)).astype(np.float32)
-    wa, wb = bf(1 + 0.2 * rng.normal(size=70)), bf(1 + 0.2 * rng.normal(size=70))
+    a, b = rng.normal(0, 3.0, (9, K)).astype(np.float32), rng.normal(0, 0.1, (9, K)).astype(np.float32)
+    wa, wb = bf(1 + 0.2 * rng.normal(size=K)), bf(1 + 0.2 * rng.normal(size=K))
     wide = dev(np.concatenate([a, a], 1))
-    got = so.rmsnorm_pair(wide[:, 70:], dev(wa, torch.bfloat16), dev(b), dev(wb, torch.bfloat16), 0.5, 1e-5)
+    got = so.rmsnorm_pair(wide[:, K:], dev(wa, torch.bfloat16), dev(b), dev(wb, torch.bfloat16), 0.5, 1e-5)
     assert rel_err(got.cpu().numpy(), 0.5 * (of.unit_rms(a, 1e-5) * wa + of.unit_rms(b, 1e-5) * wb)) < 3e-6
+
+
+@pytest.mark.parametrize("heads,P,groups", [(3, 20, 2), (64, 64, 1), (64, 64, 4), (40, 250, 1), (70, 256, 1), (70, 256, 7)])
+def test_skip_gate_and_grouped_norm(so, heads, P, groups):
+    """v = (o + D[head] x) silu(z), every one of `groups` equal parts of the row divided by its own root mean square, times the weight"""
+    rng = np.random.default_rng(3)
+    T, n = 7, heads * P
+    o, x, z = (rng.normal(0, 1.2, (T, n)).astype(np.float32) for _ in range(3))
+    skip, w = bf(rng.normal(size=heads)), bf(1 + 0.2 * rng.normal(size=n))
+    v = (o.astype(np.float64) + np.repeat(skip.astype(np.float64), P)[None] * x) * of.silu(z.astype(np.float64))
+    parts = v.reshape(T, groups, n // groups)
+    want = (parts / np.sqrt((parts ** 2).mean(-1, keepdims=True) + 1e-5)).reshape(T, n) * w
+    got = so.gate_group_rmsnorm(dev(o), dev(z), dev(w, torch.bfloat16), 1e-5, heads, P, groups, x=dev(x), skip=dev(skip, torch.bfloat16))
+    assert rel_err(got.cpu().numpy(), want) < 3e-6
+    plain = so.gate_group_rmsnorm(dev(o), dev(z), dev(w), 1e-5, heads, P, groups)         # no skip term
+    v0 = (o.astype(np.float64) * of.silu(z.astype(np.float64))).reshape(T, groups, n // groups)
+    assert rel_err(plain.cpu().numpy(), (v0 / np.sqrt((v0 ** 2).mean(-1, keepdims=True) + 1e-5)).reshape(T, n) * w) < 3e-6
 
 
 # ---------------------------------------------------------------------------------------------------------------- latent attention
